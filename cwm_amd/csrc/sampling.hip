@@ -18,6 +18,9 @@
 // with f(t*) <= top_p * sum(e); t* is found by bisection on the bit pattern.
 // Entries exactly equal to the threshold are all kept.
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 CWM_DEFINE_ERROR_API
 
@@ -212,6 +215,49 @@ extern "C" int cwm_sample(const float* logits, long row_stride, int n_rows, int 
   hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, row_stride, vocab,
                      temperature, top_p, uniform, workspace, token_out, logprob_out, sample_logprob_out);
   return cwm_launch_status("sample");
+}
+
+// ---- the same without a workspace argument: nothing is allocated ------------------ //
+// The unnormalised probabilities go to a device array of this file; see no_alloc.h.
+// In host code `sample_scratch` is only a stand-in for the symbol: its device address
+// differs from GPU to GPU and is looked up once per device, with that device current.
+static __device__ __align__(256) float sample_scratch[CWM_SAMPLE_STATIC_MAX_FLOATS];
+
+#define CWM_MAX_DEVICES 64
+static float* sample_scratch_ptr[CWM_MAX_DEVICES] = {nullptr};
+static std::mutex sample_scratch_mutex;
+
+extern "C" long cwm_sample_static_capacity() { return CWM_SAMPLE_STATIC_MAX_FLOATS; }
+
+extern "C" int cwm_sample_static(const float* logits, long row_stride, int n_rows, int vocab,
+                                 const float* temperature, const float* top_p, const float* uniform,
+                                 int* token_out, float* logprob_out, float* sample_logprob_out,
+                                 hipStream_t stream) {
+  CWM_REQUIRE(n_rows >= 0 && vocab > 0, "sample_static: bad sizes rows=%d vocab=%d", n_rows, vocab);
+  CWM_REQUIRE(row_stride >= vocab, "sample_static: row stride shorter than the vocabulary");
+  CWM_REQUIRE((long long)n_rows * vocab <= (long long)CWM_SAMPLE_STATIC_MAX_FLOATS,
+              "sample_static: %d rows of %d logits need %lld floats of scratch, the fixed array holds %d", n_rows, vocab,
+              (long long)n_rows * vocab, CWM_SAMPLE_STATIC_MAX_FLOATS);
+  if (n_rows == 0) return 0;
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess) return cwm_fail("sample_static: hipGetDevice failed: %s", hipGetErrorString(err));
+  CWM_REQUIRE(device >= 0 && device < CWM_MAX_DEVICES, "sample_static: device %d is outside 0..%d", device, CWM_MAX_DEVICES - 1);
+  float* scratch = nullptr;
+  {
+    std::lock_guard<std::mutex> guard(sample_scratch_mutex);
+    if (sample_scratch_ptr[device] == nullptr) {
+      void* found = nullptr;
+      err = hipGetSymbolAddress(&found, HIP_SYMBOL(sample_scratch));
+      if (err != hipSuccess || found == nullptr)
+        return cwm_fail("sample_static: the scratch array has no address on device %d: %s", device, hipGetErrorString(err));
+      sample_scratch_ptr[device] = (float*)found;
+    }
+    scratch = sample_scratch_ptr[device];
+  }
+  hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, row_stride, vocab,
+                     temperature, top_p, uniform, scratch, token_out, logprob_out, sample_logprob_out);
+  return cwm_launch_status("sample_static");
 }
 
 // log softmax(logits[rows[i]])[targets[i]] for given tokens: the log-probabilities of a
