@@ -112,6 +112,24 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) { return pack2
 
 extern "C" int cwm_attention_mfma_head_dim() { return HEAD_DIM; }
 
+__device__ __forceinline__ float not_a_number() { return __uint_as_float(0x7fc00000u); }
+
+// Whether any key of [first_key, last_key] (a wavefront's span, the same for all its lanes) lies in a
+// logical page whose table entry is no page of the pool: the lanes test the entries side by side.
+__device__ __forceinline__ bool span_lacks_page(const int* __restrict__ table, int table_width, int num_pages,
+                                                int page_size, int page_shift, int first_key, int last_key, int lane) {
+  bool bad = false;
+  if (last_key >= first_key && first_key >= 0) {
+    const int lp_first = page_shift >= 0 ? (first_key >> page_shift) : (first_key / page_size);
+    const int lp_last = page_shift >= 0 ? (last_key >> page_shift) : (last_key / page_size);
+    for (int lp = lp_first + lane; lp <= lp_last; lp += 64) {
+      const int page = lp < table_width ? table[lp] : -1;
+      bad = bad || (unsigned)page >= (unsigned)num_pages;
+    }
+  }
+  return __any(bad);
+}
+
 // work item: {sequence, first row, first key, end key (exclusive), partial slot or -1, unused}
 // One wavefront per (work item, key/value head); RT: 16-row tiles that a wavefront takes from
 // the item's first row on.  Decoded tokens and short portions run with RT = 1 (sequences with
@@ -220,6 +238,9 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __res
   const int* table = block_table + (size_t)b * table_width;
   const bf16_t* kbase = cache + (size_t)g * page_size * HEAD_DIM;
   const bf16_t* vbase = cache + plane + (size_t)g * page_size * HEAD_DIM;
+  // a key that some row reads must have a page: if its table entry is -1 or out of range the rows'
+  // results are made NaN (the loads below then read page 0, so nothing faults)
+  const bool page_missing = span_lacks_page(table, table_width, num_pages, page_size, page_shift, lo_any, hi_any, lane);
 
   // page of a key; keys outside [0, key_end) and slots without a page read page 0 and are masked
   auto page_of = [&](int key, int& slot_in_page) -> int {
@@ -353,7 +374,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __res
     if (!row_valid[rt]) continue;
     if (slot < 0) {
       // the whole key range was this wavefront's: normalise and store
-      const float inv = 1.0f / l_row;
+      const float inv = page_missing ? not_a_number() : 1.0f / l_row;
       bf16_t* orow = out + (size_t)(q0 + ti[rt]) * out_stride + (size_t)hq[rt] * HEAD_DIM;
 #pragma unroll
       for (int dt = 0; dt < D_TILES; ++dt) {
@@ -369,7 +390,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __res
       for (int dt = 0; dt < D_TILES; ++dt) *(float4v*)(prow + 16 * dt + 4 * j) = acc[rt][dt];
       if (j == 0) {
         prow[HEAD_DIM] = m_run[rt] * scale_log2e;  // the merge works in the scaled (log2) domain
-        prow[HEAD_DIM + 1] = l_row;
+        prow[HEAD_DIM + 1] = page_missing ? not_a_number() : l_row;  // the merged row becomes NaN too
       }
     }
   }
@@ -636,6 +657,10 @@ attention_lds_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __rest
     hi_all = rt == 0 ? hi_a : min(hi_all, hi_a);
   }
 
+  // a key that a row of this wavefront reads must have a page, or the wavefront's rows become NaN
+  const bool page_missing =
+      span_lacks_page(table, table_width, num_pages, page_size, page_shift, max(lo_w, key_begin), min(hi_w, key_end - 1), lane);
+
   // one 32-key tile from LDS buffer `buf`: scores, running softmax, weighted values
   auto compute = [&](int kt, const bf16_t* kbuf, const bf16_t* vbuf) {
     // a wavefront whose rows all end before this tile, or start after it, has nothing to add
@@ -853,11 +878,11 @@ attention_lds_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __rest
       for (int dt = 0; dt < D_TILES; ++dt) *(float4v*)(prow + 16 * dt + 4 * j) = acc[rt][dt];
       if (j == 0) {
         prow[HEAD_DIM] = m_run[rt] * scale_log2e;
-        prow[HEAD_DIM + 1] = l_row;
+        prow[HEAD_DIM + 1] = page_missing ? not_a_number() : l_row;
       }
       continue;
     }
-    const float inv = 1.0f / l_row;
+    const float inv = page_missing ? not_a_number() : 1.0f / l_row;
     bf16_t* orow = out + (size_t)(q0 + ti[rt]) * out_stride + (size_t)hq[rt] * HEAD_DIM;
 #pragma unroll
     for (int dt = 0; dt < D_TILES; ++dt) {

@@ -16,6 +16,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager
+from ..cache.pages import first_page_needed, pages_for
 
 
 @dataclass
@@ -126,6 +127,15 @@ def build_batch(
             pages = manager.table(g.index, rid)
             n = min(len(pages), width)
             tbl[b, :n] = pages[:n]
+            # every page that this step's queries can read, or that its tokens are written to, is held
+            first = first_page_needed(kv_lens[b] - q_lens[b], g.window, page_size)
+            last = pages_for(kv_lens[b], page_size)
+            span = tbl[b, first:last]
+            if span.size != last - first or (span < 0).any() or (span >= g.pool.num_pages).any():
+                raise BatchError(
+                    f"request {rid!r}: group {g.index} holds no page for some of the logical pages {first}..{last - 1} "
+                    f"that this step reads or writes (table {span.tolist()}, pool of {g.pool.num_pages})"
+                )
         tables.append(tbl)
 
     # one buffer, one copy

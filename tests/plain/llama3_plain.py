@@ -4,6 +4,18 @@ Each function is written from the text of the reference (file:line cited in its
 docstring), operates on whole sequences with no cache, and imports nothing from
 the product package.  All arithmetic runs in the dtype of the inputs (tests use
 float32 or float64 on the CPU).
+
+`forward(..., rounding=...)` also emulates a bfloat16 run: the arithmetic stays in
+the wide type and the value is rounded to bfloat16 at the places where a
+bfloat16 run stores it.  `ROUND_AS_REFERENCE` rounds where the reference does
+(every tensor it keeps is bfloat16: cwm/fastgen/forward.py:543-546 embedding, :571
+and :772,789 norm outputs, :593-606 projections, :618-619 rotated q and k, :639-655
+attention output, :763,769 output projection and the residual sum, :776-781 both
+branches, silu and the product, :782,786 down projection and residual sum,
+:820-821 logits); `ROUND_AS_ENGINE` rounds where the engine under test keeps a
+bfloat16 tensor (the residual stream and the logits stay wide, silu(gate) * up
+is rounded once).  In both, the attention probabilities are rounded before
+the product with the values, as a matrix-core attention kernel has to.
 """
 
 from __future__ import annotations
@@ -55,6 +67,10 @@ def window_left_of_layer(
         return -1 if gw is None else int(gw) - 1
     lw = window_attn.get("local_window")
     return -1 if lw is None else int(lw) - 1
+
+
+ROUND_AS_REFERENCE = "reference"
+ROUND_AS_ENGINE = "engine"
 
 
 # --------------------------------------------------------------------------- #
@@ -124,41 +140,66 @@ def rope_apply(x: torch.Tensor, positions: torch.Tensor, freqs: torch.Tensor) ->
     return out
 
 
+def round_bf16(x: torch.Tensor) -> torch.Tensor:
+    """x rounded to the nearest bfloat16 (ties to even), in x's own type."""
+    return x.to(torch.bfloat16).to(x.dtype)
+
+
 def attention(
     q: torch.Tensor,
     k: torch.Tensor,
     v: torch.Tensor,
     window_left: int = -1,
     scale: Optional[float] = None,
+    round_probabilities: bool = False,
 ) -> torch.Tensor:
     """Causal grouped-query attention over one whole sequence.
 
     cwm/fastgen/forward.py:638-655: softmax(q k^T * hd^-1/2) v over keys j <= p and,
     with window_left = w >= 0, j >= p - w; query head h reads key/value head
     h // (Hq / Hkv).  q: [T, Hq, hd]; k, v: [T, Hkv, hd]; returns [T, Hq, hd].
+    With `round_probabilities` the unnormalised probabilities exp(s - max) are
+    rounded to bfloat16 for the sum over the values while their own sum is not, as
+    in an attention kernel that feeds them to a bfloat16 matrix product.
     """
     n_tok, n_q, hd = q.shape
     n_kv = k.shape[1]
     group = n_q // n_kv
     if scale is None:
         scale = hd ** -0.5
+    pos = torch.arange(n_tok)
+    distance = pos[:, None] - pos[None, :]  # query position - key position
+    allowed = distance >= 0
+    if window_left >= 0:
+        allowed &= distance <= window_left
     out = torch.empty_like(q)
     for h in range(n_q):
         g = h // group
         scores = (q[:, h, :] @ k[:, g, :].T) * scale  # [T, T]
-        for p in range(n_tok):
-            lo = 0 if window_left < 0 else max(0, p - window_left)
-            s = scores[p, lo : p + 1]
-            w = torch.softmax(s, dim=-1)
-            out[p, h, :] = w @ v[lo : p + 1, g, :]
+        scores = scores.masked_fill(~allowed, float("-inf"))
+        if round_probabilities:
+            e = torch.exp(scores - scores.max(dim=-1, keepdim=True).values)
+            out[:, h, :] = (round_bf16(e) @ v[:, g, :]) / e.sum(dim=-1, keepdim=True)
+        else:
+            out[:, h, :] = torch.softmax(scores, dim=-1) @ v[:, g, :]
     return out
 
 
-def swiglu(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor) -> torch.Tensor:
-    """(silu(x w1^T) * (x w3^T)) w2^T.  cwm/fastgen/forward.py:776-782."""
-    gate = x @ w1.T
-    up = x @ w3.T
-    return (gate * torch.sigmoid(gate) * up) @ w2.T
+def swiglu(
+    x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor, rounding: Optional[str] = None
+) -> torch.Tensor:
+    """(silu(x w1^T) * (x w3^T)) w2^T.  cwm/fastgen/forward.py:776-782.
+
+    In a bfloat16 run the reference stores x1, x3, silu(x1) (in place) and the
+    product (in place), each rounded (:776-781); the engine stores both branches
+    and the finished product."""
+    rnd = round_bf16 if rounding else (lambda t: t)
+    gate = rnd(x @ w1.T)
+    up = rnd(x @ w3.T)
+    act = gate * torch.sigmoid(gate)
+    if rounding == ROUND_AS_REFERENCE:
+        act = rnd(act)
+    return rnd(rnd(act * up) @ w2.T)
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -185,6 +226,7 @@ def forward(
     window_left: Sequence[int],
     first_position: int = 0,
     dtype: torch.dtype = torch.float32,
+    rounding: Optional[str] = None,
 ) -> torch.Tensor:
     """Logits [T, V] of one whole sequence.
 
@@ -193,34 +235,48 @@ def forward(
     h += w2(silu(w1 x) * w3 x) with x = norm(h); final norm; output projection.
     Weight names are the module names of cwm/model/transformer.py:173-193,214-228,
     244-252,301-313.  `first_position` shifts every position (used by tests of the
-    rotation's dependence on distances only).
+    rotation's dependence on distances only).  `rounding`: None, or one of
+    ROUND_AS_REFERENCE / ROUND_AS_ENGINE (see the module's text): the weights are
+    rounded to bfloat16 and so is every tensor that such a run stores.
     """
+    if rounding not in (None, ROUND_AS_REFERENCE, ROUND_AS_ENGINE):
+        raise ValueError(f"unknown rounding {rounding!r}")
+    rnd = round_bf16 if rounding else (lambda t: t)
+    # the residual stream: bfloat16 in the reference (h.add_ at forward.py:769,786), wide in the engine
+    rnd_h = round_bf16 if rounding == ROUND_AS_REFERENCE else (lambda t: t)
+    weights = {name: (t.to(torch.bfloat16) if rounding and t.is_floating_point() else t) for name, t in weights.items()}
     w = {name: t.to(dtype) for name, t in weights.items()}
     tok = torch.as_tensor(list(tokens), dtype=torch.long)
     positions = torch.arange(len(tok)) + first_position
     h = w["tok_embeddings.weight"][tok]
     for i in range(n_layers):
         pre = f"layers.{i}."
-        x = rms_norm(h, w[pre + "attention_norm.weight"], norm_eps)
-        xq = linear(x, w[pre + "attention.wq.weight"], w.get(pre + "attention.wq.bias"))
-        xk = linear(x, w[pre + "attention.wk.weight"], w.get(pre + "attention.wk.bias"))
-        xv = linear(x, w[pre + "attention.wv.weight"], w.get(pre + "attention.wv.bias"))
+        x = rnd(rms_norm(h, w[pre + "attention_norm.weight"], norm_eps))
+        xq = rnd(linear(x, w[pre + "attention.wq.weight"], w.get(pre + "attention.wq.bias")))
+        xk = rnd(linear(x, w[pre + "attention.wk.weight"], w.get(pre + "attention.wk.bias")))
+        xv = rnd(linear(x, w[pre + "attention.wv.weight"], w.get(pre + "attention.wv.bias")))
         xq = xq.view(-1, n_heads, head_dim)
         xk = xk.view(-1, n_kv_heads, head_dim)
         xv = xv.view(-1, n_kv_heads, head_dim)
-        xq = rope_apply(xq, positions, rope_freqs)
-        xk = rope_apply(xk, positions, rope_freqs)
-        att = attention(xq, xk, xv, window_left=window_left[i])
-        h = h + linear(att.reshape(len(tok), -1), w[pre + "attention.wo.weight"])
-        x = rms_norm(h, w[pre + "ffn_norm.weight"], norm_eps)
-        h = h + swiglu(
-            x,
-            w[pre + "feed_forward.w1.weight"],
-            w[pre + "feed_forward.w2.weight"],
-            w[pre + "feed_forward.w3.weight"],
+        xq = rnd(rope_apply(xq, positions, rope_freqs))
+        xk = rnd(rope_apply(xk, positions, rope_freqs))
+        att = rnd(attention(xq, xk, xv, window_left=window_left[i], round_probabilities=bool(rounding)))
+        h = rnd_h(h + rnd(linear(att.reshape(len(tok), -1), w[pre + "attention.wo.weight"])))
+        x = rnd(rms_norm(h, w[pre + "ffn_norm.weight"], norm_eps))
+        h = rnd_h(
+            h
+            + swiglu(
+                x,
+                w[pre + "feed_forward.w1.weight"],
+                w[pre + "feed_forward.w2.weight"],
+                w[pre + "feed_forward.w3.weight"],
+                rounding,
+            )
         )
-    h = rms_norm(h, w["norm.weight"], norm_eps)
-    return linear(h, w["output.weight"])
+    h = rnd(rms_norm(h, w["norm.weight"], norm_eps))
+    logits = linear(h, w["output.weight"])
+    # the reference's head writes bfloat16 before `.float()` (forward.py:820-821); the engine's writes float32
+    return round_bf16(logits) if rounding == ROUND_AS_REFERENCE else logits
 
 
 def forward_from_config(
@@ -229,6 +285,7 @@ def forward_from_config(
     tokens: Sequence[int],
     dtype: torch.dtype = torch.float32,
     first_position: int = 0,
+    rounding: Optional[str] = None,
 ) -> torch.Tensor:
     """`forward` with its constants taken from a config.json dictionary.
 
@@ -272,6 +329,7 @@ def forward_from_config(
         window_left=lefts,
         first_position=first_position,
         dtype=dtype,
+        rounding=rounding,
     )
 
 

@@ -12,7 +12,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import configs, generation, models, traces
+from helpers import compare as cmp, configs, generation, models, traces
 
 pytestmark = pytest.mark.gpu
 
@@ -90,10 +90,9 @@ def test_trace_run_program(tmp_path):
             else:
                 assert not f.exists()
         got = traces.gather(steps, outputs, {k: len(v) for k, v in requests.items()}, vocab)
-        want = models.plain_logits(folder, requests)
-        limit = 3e-5 if dtype == "float32" else 4e-2
+        want = cmp.expected(folder, requests, dtype)
         for rid in requests:
-            assert np.abs(got[rid] - want[rid]).max() <= limit * np.abs(want[rid]).max()
+            cmp.check(got[rid], want[rid], dtype, f"trace_run {dtype} {rid}")
 
 
 # ---- a toy mixer with state of its own -------------------------------------------------- #

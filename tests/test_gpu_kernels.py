@@ -467,6 +467,70 @@ def test_attention_mfma_long_ranges(window):
     torch.testing.assert_close(got.float(), torch.cat(want_rows), rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("n_q,n_kv,hd,page_size", [(6, 2, 64, 32), (12, 2, 128, 64), (6, 3, 48, 8)])
+def test_missing_page_shows_as_nan_in_both_attention_kernels(n_q, n_kv, hd, page_size):
+    """A block-table entry of -1 (or past the pool) for a page that a query reads must not pass
+    for page 0: every row that reads it comes out NaN, from the matrix-core kernels (decoded
+    token, split and merged; short portion; long portion through LDS, with and without direct
+    loads) as from the plain kernel; rows of other sequences, and rows whose window has passed
+    the page, stay finite."""
+    from types import SimpleNamespace
+
+    from cwm_amd import ops
+
+    dtype = torch.bfloat16
+    lens_old, lens_new = [2000, 100, 0, 40, 900], [1, 1, 300, 5, 1]
+    n_seqs = len(lens_old)
+    kv_lens = [a + b for a, b in zip(lens_old, lens_new)]
+    width = max((n + page_size - 1) // page_size for n in kv_lens)
+    total_pages = sum((n + page_size - 1) // page_size for n in kv_lens)
+    table = torch.full((n_seqs, width), -1, dtype=torch.int32)
+    used = 0
+    for b, n in enumerate(kv_lens):
+        n_pages = (n + page_size - 1) // page_size
+        table[b, :n_pages] = torch.arange(used, used + n_pages, dtype=torch.int32)
+        used += n_pages
+    g = torch.Generator().manual_seed(3)
+    cache = torch.randn((total_pages, 2, n_kv, page_size * hd), generator=g).to(dtype).to(DEV)
+    q = torch.randn((sum(lens_new), n_q, hd), generator=g).to(dtype).to(DEV)
+    cu = [0]
+    for n in lens_new:
+        cu.append(cu[-1] + n)
+    positions = torch.cat([torch.arange(a, a + b) for a, b in zip(lens_old, lens_new)]).to(torch.int32).to(DEV)
+    seq_of = torch.cat([torch.full((n,), b) for b, n in enumerate(lens_new)]).to(torch.int32).to(DEV)
+
+    def run(tbl, window):
+        batch = SimpleNamespace(
+            q_lens=lens_new, kv_lens=kv_lens, n_seqs=n_seqs, n_tokens=sum(lens_new), scratch={},
+            cu_q=torch.tensor(cu, dtype=torch.int32).to(DEV), kv_len=torch.tensor(kv_lens, dtype=torch.int32).to(DEV),
+        )
+        mfma = ops.paged_attention_mfma(q, cache, tbl.to(DEV), batch, window, hd ** -0.5).float().cpu()
+        simple = ops.paged_attention_simple(q, cache, tbl.to(DEV), positions, seq_of, window, hd ** -0.5).float().cpu()
+        return mfma, simple
+
+    for out in run(table, None):
+        assert torch.isfinite(out).all()
+    # no window: everyone reads logical page 0 of their sequence
+    for b in range(n_seqs):
+        broken = table.clone()
+        broken[b, 0] = -1 if b % 2 == 0 else total_pages + 5
+        for name, out in zip(("matrix-core", "plain"), run(broken, None)):
+            rows = slice(cu[b], cu[b + 1])
+            assert torch.isnan(out[rows]).all(), f"{name}: sequence {b} read a missing page and shows no NaN"
+            rest = torch.cat([out[: cu[b]], out[cu[b + 1] :]])
+            assert torch.isfinite(rest).all(), f"{name}: a missing page of sequence {b} reached other sequences"
+    # a window of 70 keys: page 0 of the long sequences is out of reach, the page of key 1,960 is not
+    window = 70
+    broken = table.clone()
+    broken[0, 0] = -1
+    broken[4, 0] = -1
+    for name, out in zip(("matrix-core", "plain"), run(broken, window)):
+        assert torch.isfinite(out).all(), f"{name}: a page that the window has passed was read"
+    broken[0, 1960 // page_size] = -1
+    for name, out in zip(("matrix-core", "plain"), run(broken, window)):
+        assert torch.isnan(out[0]).all() and torch.isfinite(out[1:]).all(), name
+
+
 def test_attention_mfma_builds_agree_bit_for_bit(monkeypatch):
     """The wrapper picks between builds of the same arithmetic by the shape of the work (two or
     three blocks a compute unit for long portions; the wavefront index declared uniform or not

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import configs, models, traces
+from helpers import compare as cmp, configs, models, traces
 
 pytestmark = pytest.mark.gpu
 
@@ -23,21 +23,9 @@ def requests_for(name):
     return {f"r{i}": traces.random_tokens(7 * i + len(name), n, vocab) for i, n in enumerate(LENGTHS[name])}
 
 
-def limits(dtype):
-    # largest error over a request's logits, relative to the largest logit
-    return 3e-5 if dtype == "float32" else 4e-2
-
-
 def compare(got, want, dtype, what):
     for rid in want:
-        assert not np.isnan(got[rid]).any(), f"{what} {rid}: missing or NaN logits"
-        err = np.abs(got[rid] - want[rid]).max(axis=1)
-        scale = np.abs(want[rid]).max()
-        worst = int(err.argmax())
-        assert err.max() <= limits(dtype) * scale, (
-            f"{what} {rid}: first position over the limit {int(np.argmax(err > limits(dtype) * scale))}, "
-            f"worst position {worst} error {err.max():.3e} vs scale {scale:.3e}"
-        )
+        cmp.check(got[rid], want[rid], dtype, f"{what} {rid}")
 
 
 @pytest.fixture(scope="module")
@@ -58,7 +46,7 @@ def plain_cache():
 def plain_for(folders, plain_cache, name, dtype):
     key = (name, dtype)
     if key not in plain_cache:
-        plain_cache[key] = models.plain_logits(folders[key], requests_for(name), dtype=torch.float64)
+        plain_cache[key] = cmp.expected(folders[key], requests_for(name), dtype)
     return plain_cache[key]
 
 
@@ -93,7 +81,7 @@ def test_first_tokens_and_long_decoding(folders, plain_cache, dtype):
     rep = Replayer(folders[name, dtype], dtype, 320, page_size=4, poison_freed_pages=True)
     outputs = traces.run_in_process(rep, steps)
     got = traces.gather(steps, outputs, {"x": len(toks)}, vocab)
-    want = models.plain_logits(folders[name, dtype], {"x": toks})
+    want = cmp.expected(folders[name, dtype], {"x": toks}, dtype)
     compare(got, want, dtype, f"{name} {dtype} one-by-one")
     # the window group never holds more than the window needs
     local = [g.index for g in rep.manager.groups if g.window is not None]

@@ -39,3 +39,34 @@ def test_regimes_against_plain(tmp_path, monkeypatch, name, lengths, regime):
         np.testing.assert_allclose(got[rid], want[rid], rtol=2e-4, atol=2e-5, err_msg=f"{name} {regime} {rid}")
     assert rep.manager.live_requests() == []
     assert all(f == g.pool.num_pages for f, g in zip(rep.manager.free_pages(), rep.manager.groups))
+
+
+def test_a_step_whose_readable_pages_are_not_all_held_is_refused():
+    """The descriptor is refused when a logical page that the step's queries read, or that its
+    tokens are written to, has no page of the pool; a page that the window has passed may be gone."""
+    from cwm_amd.cache import CacheManager
+    from cwm_amd.engine.batch import BatchError, Portion, build_batch
+    from cwm_amd.parts import PagedKVSpec
+
+    specs = [PagedKVSpec(1, 16, None), PagedKVSpec(1, 16, 6)]
+    manager = CacheManager(specs, 4, 16, 2)
+    manager.admit("a")
+    assert manager.extend("a", 20)
+    manager.advance("a", 20)  # the window group has given back pages 0..2 (keys 0..11 lie before 20 - 5)
+    assert manager.table(1, "a")[:3] == [-1, -1, -1]
+    assert manager.extend("a", 3)
+    device = torch.device("cpu")
+    build_batch([Portion("a", [1, 2, 3], [2])], manager, device, 50)  # fine as it is
+    # a hole where the first query of the portion still reads (key 15 = 20 - 5 lies in page 3)
+    held = manager.table(1, "a")[3]
+    manager.table(1, "a")[3] = -1
+    with pytest.raises(BatchError, match="holds no page"):
+        build_batch([Portion("a", [1, 2, 3], [2])], manager, device, 50)
+    manager.table(1, "a")[3] = held
+    # a hole in the keep-all group, far back
+    held = manager.table(0, "a")[0]
+    manager.table(0, "a")[0] = 99
+    with pytest.raises(BatchError, match="holds no page"):
+        build_batch([Portion("a", [1, 2, 3], [2])], manager, device, 50)
+    manager.table(0, "a")[0] = held
+    build_batch([Portion("a", [1, 2, 3], [2])], manager, device, 50)
