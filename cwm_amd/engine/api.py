@@ -34,6 +34,8 @@ class GenArgs:
     min_prefill: int = 512  # reference batching threshold: not needed with mixed steps, ignored
     min_prefill_batch: int = 8  # likewise ignored
 
+    expected_seq: int = -1  # not in the reference: tokens a typical request holds; how free memory is split between
+    # layer groups when max_seq is negative (negative: the context length the model's configuration names)
     prefill_gb: float = 2  # memory kept free for activations when max_seq is negative
     gpu_gb: float = 74  # the reference's memory budget: ignored, free memory is measured
 

@@ -14,6 +14,7 @@ control back.
 
 from __future__ import annotations
 
+import os
 import queue
 import time
 from typing import Any, Dict, Generator, Iterable, List, Optional, Sequence, Union
@@ -27,18 +28,35 @@ from ..parts.base import PagedKVSpec
 from ..sampling.sampler import RequestStream, Sampler, effective_temperature
 from .api import GenArgs, Packet
 from .loading import load_model, random_model
+from .metrics import MetricsLog
 from .runner import ModelRunner
 from .scheduler import Request, Scheduler
 
 
-def pool_sizes(model: Model, args: GenArgs, device: torch.device) -> Dict[Optional[int], int]:
-    """Pages of every layer group.
+def pool_sizes(
+    model: Model,
+    args: GenArgs,
+    device: torch.device,
+    free_bytes: Optional[int] = None,
+) -> Dict[Optional[int], int]:
+    """Pages of every layer group (keyed by the group's window, None for the group that keeps
+    all keys).
 
-    The group that keeps all keys gets `max_seq` tokens (cwm/fastgen/generate.py:
-    245-251); a negative `max_seq` takes what free memory allows after a reserve for
-    activations (the rule of cwm/fastgen/utils/tune.py:90-107 with measured free
-    memory).  A group whose layers read a window W never needs more than
-    W - 1 + max_prefill tokens (plus a page of slack at either end) per request.
+    With `max_seq` given, the keep-all group holds that many tokens
+    (cwm/fastgen/generate.py:245-251) and a group with window W the same, or less if
+    `max_batch` requests cannot fill it: a request never holds more than W - 1 + max_prefill
+    tokens there (plus a page of slack at either end).
+
+    With a negative `max_seq` the pools share what is free on the device after a reserve for
+    activations (the reference's rule, cwm/fastgen/utils/tune.py:90-107, which knows one pool
+    only).  The split follows what one expected request needs of each group: `expected_seq`
+    tokens of the keep-all group against min(expected_seq, W - 1 + max_prefill) of a window
+    group; `expected_seq` defaults to the context length that the model's configuration
+    names.  Without either, every group gets room for the same number of tokens.  A window
+    group is never made larger than `max_batch` requests can fill; what that saves goes to the
+    keep-all group.  No pool is sized for the worst case of `max_batch` requests up front:
+    when any group runs out of pages the scheduler preempts, whichever group it is.
+    `free_bytes` stands in for the measured free memory (tests).
     """
     page = args.cache_block
     esize = 4 if model.runtime.act_dtype == torch.float32 else 2
@@ -46,34 +64,50 @@ def pool_sizes(model: Model, args: GenArgs, device: torch.device) -> Dict[Option
     for spec in model.cache_specs:
         if isinstance(spec, PagedKVSpec):
             per_page[spec.window] = per_page.get(spec.window, 0) + 2 * spec.n_kv_heads * spec.head_dim * page * esize
+    if not per_page:
+        return {}
+
+    def request_cap(window: int) -> int:
+        """Most pages that `max_batch` requests can hold of a window group."""
+        return args.max_batch * ((window - 1 + args.max_prefill + page - 1) // page + 2)
+
     sizes: Dict[Optional[int], int] = {}
-    windows = sorted((w for w in per_page if w is not None))
-    cap_tokens = args.max_seq if args.max_seq > 0 else None
-    local_bytes = 0
-    for w in windows:
-        pages = args.max_batch * ((w - 1 + args.max_prefill + page - 1) // page + 2)
-        if cap_tokens is not None:
-            pages = min(pages, (cap_tokens + page - 1) // page)
-        sizes[w] = max(1, pages)
-        local_bytes += sizes[w] * per_page[w]
-    if cap_tokens is not None:
+    if args.max_seq > 0:
+        cap_pages = (args.max_seq + page - 1) // page
         for w in per_page:
-            if w is None or w not in sizes:
-                sizes[w] = max(1, (cap_tokens + page - 1) // page)
+            sizes[w] = max(1, cap_pages if w is None else min(request_cap(w), cap_pages))
         return sizes
-    if device.type != "cuda":
-        raise ValueError("max_seq must be given when no HIP device is used")
+
+    if free_bytes is None:
+        if device.type != "cuda":
+            raise ValueError("max_seq must be given when no HIP device is used")
+        free_bytes, _total = torch.cuda.mem_get_info(device)
     # nine tenths of what is free after the reserve: the rest is slack for the allocator
-    free, _total = torch.cuda.mem_get_info(device)
-    budget = int(0.9 * (free - int(args.prefill_gb * 1e9))) - local_bytes
-    if None in per_page:
-        sizes[None] = budget // per_page[None]
-        if sizes[None] < args.max_batch:
-            raise MemoryError(
-                f"free memory leaves room for {sizes[None]} pages of {page} tokens, fewer than max_batch={args.max_batch}"
-            )
-    elif budget < 0:
-        raise MemoryError("the windows' pages alone do not fit into free memory; lower max_batch or max_prefill")
+    budget = int(0.9 * (free_bytes - int(args.prefill_gb * 1e9)))
+    expected = args.expected_seq if args.expected_seq > 0 else (model.plan.max_positions or 0)
+    # pages that one expected request holds of each group
+    share: Dict[Optional[int], int] = {}
+    for w in per_page:
+        if expected <= 0:
+            share[w] = 1
+        else:
+            tokens = expected if w is None else min(expected, w - 1 + args.max_prefill)
+            share[w] = (tokens + page - 1) // page + 1
+    per_request = sum(share[w] * per_page[w] for w in per_page)
+    requests = budget / per_request if budget > 0 else 0.0
+    for w in per_page:
+        sizes[w] = int(requests * share[w])
+        if w is not None and sizes[w] > request_cap(w):
+            sizes[w] = request_cap(w)
+    if None in per_page:  # what the caps saved
+        rest = budget - sum(sizes[w] * per_page[w] for w in per_page if w is not None)
+        sizes[None] = max(sizes[None], rest // per_page[None])
+    smallest = min(sizes.values())
+    if smallest < 1:
+        raise MemoryError(
+            f"{free_bytes / 1e9:.1f} GB of free memory less {args.prefill_gb} GB for activations leave no room for "
+            f"one page of {page} tokens in every layer group (bytes per page: {per_page})"
+        )
     return sizes
 
 
@@ -97,8 +131,20 @@ class Engine:
         self.manager = CacheManager(model.cache_specs, args.cache_block, sizes, args.max_batch)
         self.storage = CacheStorage(self.manager, self.device, model.runtime.act_dtype)
         self.runner = ModelRunner(model, self.manager, self.storage)
-        self.scheduler = Scheduler(self.manager, args.max_batch, args.max_prefill)
+        # a request joins others only when its known tokens and some room to decode fit
+        # (the reference asks for 128 tokens of room, cwm/fastgen/generate.py:596-597)
+        self.scheduler = Scheduler(self.manager, args.max_batch, args.max_prefill, headroom=min(128, args.cache_block))
         self.sampler = Sampler(self.device)
+        self.metrics = MetricsLog()
+        self.scheduler.on_event = self._scheduler_event
+        self._last_active = 0
+        # a window of traced steps (cwm/fastgen/generate.py:148-156,397-434)
+        self._profile_state = "inactive"
+        self._profile_iter = 0
+        self._profile_ctx: Any = None
+        self.profile_iters = int(os.environ.get("FG_PROFILE_ITERS", "8"))
+        self.profile_dir = os.environ.get("FG_PROFILE_DIR", "/tmp")
+        self.last_profile_path: Optional[str] = None
         if None in sizes:
             self.max_seq = sizes[None] * args.cache_block
         else:
@@ -177,17 +223,69 @@ class Engine:
             finish_reason=request.finish_reason,
         )
 
+    # ---- events and profiles ----------------------------------------------------------- #
+    def _scheduler_event(self, kind: str, request: Request) -> None:
+        if kind == "admit" and request.preemptions > 0:
+            self.metrics.record("unpark", tokens=len(request))
+        elif kind == "preempt":
+            self.metrics.record("preempt", tokens=len(request))
+
+    def request_profile(self) -> None:
+        """Trace the next `profile_iters` steps (FG_PROFILE_ITERS, default 8) with torch's
+        profiler and write a Chrome trace into `profile_dir` (FG_PROFILE_DIR, default /tmp);
+        cwm/fastgen/generate.py:397-434."""
+        if self._profile_state == "inactive":
+            self._profile_state = "requested"
+
+    def _profile_step(self) -> None:
+        if self._profile_state == "active":
+            self._profile_iter += 1
+            if self._profile_iter >= self.profile_iters:
+                self._profile_done()
+            return
+        if self._profile_state != "requested":
+            return
+        from torch.profiler import ProfilerActivity, profile
+
+        activities = [ProfilerActivity.CPU]
+        if self.device.type == "cuda":
+            activities.append(ProfilerActivity.CUDA)
+        self._profile_iter = 0
+        self._profile_ctx = profile(activities=activities)
+        self._profile_ctx.__enter__()
+        self._profile_state = "active"
+
+    def _profile_done(self) -> None:
+        if self._profile_state != "active":
+            self._profile_state = "inactive"
+            return
+        self._profile_state = "inactive"
+        ctx, self._profile_ctx = self._profile_ctx, None
+        ctx.__exit__(None, None, None)
+        path = os.path.join(self.profile_dir, f"cwm_amd_{time.strftime('%y%m%d-%H%M%S')}_{os.getpid()}.json.gz")
+        ctx.export_chrome_trace(path)
+        self.last_profile_path = path
+
     # ---- one step -------------------------------------------------------------------- #
     def step(self) -> List[Packet]:
         """Schedule, run and sample one step; returns the requests it finished."""
         sched = self.scheduler
-        already = len(sched.finished)
+        if self._profile_state != "inactive":
+            self._profile_step()
+        already = 0 if not sched.finished else len(sched.finished)
         # a request that may not grow at all is done before it starts
         for request in list(sched.waiting):
             if request.max_len <= len(request.prompt):
                 sched.waiting.remove(request)
                 sched._finish(request, "length")
         batch = sched.schedule()
+        if len(sched.running) != self._last_active:
+            self._last_active = len(sched.running)
+            if self.metrics.enabled():
+                self.metrics.record(
+                    "nactive", lanes=self._last_active, free_pages=self.manager.free_pages(),
+                    pages=[g.pool.num_pages for g in self.manager.groups],
+                )
         for item in batch:
             if item.start == 0 and item.request.cached == 0:
                 self.storage.zero_state(self.manager.slot(item.request.rid))
@@ -229,6 +327,10 @@ class Engine:
                 tokens, logprobs, sample_logprobs = [], [], []
             sched.step_done(batch, tokens, self.stop_tokens, logprobs, sample_logprobs)
         out = [self._packet(r) for r in sched.finished[already:]]
+        for packet in out:
+            self.metrics.record("yield", tokens=len(packet.tokens))
+        # what has been handed back is not kept: a long-lived generate(q) would collect every request
+        del sched.finished[:]
         return out
 
     # ---- the reference's generator interface ------------------------------------------ #
@@ -252,6 +354,7 @@ class Engine:
             iterations += 1
             if self.args.handover_frequency > 0 and iterations % self.args.handover_frequency == 0:
                 yield None
+        self._profile_done()
 
     def generate_tokens(
         self,

@@ -12,6 +12,11 @@ have gathered (:645-653); here every step takes one token from each decoding
 request first and fills the rest of the budget (`max_prefill`, :55) with prompt
 portions in arrival order, so no such threshold is needed.
 
+A request joins running ones only when every group has free pages for all of its known
+tokens and `headroom` more (the reference admits a lane when prompt + 128 tokens fit,
+:596-597,627-640): one that was let in with part of its prompt would be the shortest
+when pages run out, lose what it has computed and come back, over and over.
+
 When pages run out (`CacheManager.extend` fails):
   * for a decoding request, the shortest running request is preempted, as the
     reference parks the shortest lane (:540-566): its pages are given back, it goes
@@ -26,9 +31,10 @@ from __future__ import annotations
 
 from collections import deque
 from dataclasses import dataclass, field
-from typing import Any, Deque, Dict, Hashable, List, Optional, Sequence, Set
+from typing import Any, Callable, Deque, Dict, Hashable, List, Optional, Sequence, Set
 
 from ..cache.manager import CacheManager
+from ..cache.pages import pages_for
 from .batch import Portion
 
 WAITING, RUNNING, PARKED, FINISHED = "waiting", "running", "parked", "finished"
@@ -77,17 +83,25 @@ class Scheduled:
 
 
 class Scheduler:
-    def __init__(self, manager: CacheManager, max_batch: int, max_tokens_per_step: int) -> None:
+    def __init__(self, manager: CacheManager, max_batch: int, max_tokens_per_step: int, headroom: int = 0) -> None:
         self.manager = manager
         self.max_batch = max_batch
         self.max_tokens_per_step = max_tokens_per_step
+        self.headroom = headroom  # tokens of room to decode that a request needs beside its known tokens to join others
         self.waiting: Deque[Request] = deque()
         self.parked: Deque[Request] = deque()
         self.running: List[Request] = []
-        self.finished: List[Request] = []
+        self.finished: List[Request] = []  # the caller may empty it once it has taken what it needs
         self._arrivals = 0
         self._preempted_now = False
-        self.events: List[str] = []  # admit / preempt / finish, in order (for logs and tests)
+        self.events: Deque[str] = deque(maxlen=4096)  # the latest admit / preempt / finish events, in order
+        self.n_preemptions = 0
+        self.on_event: Optional[Callable[[str, Request], None]] = None  # called as on_event("admit" | "preempt" | "finish", request)
+
+    def _event(self, kind: str, request: Request, detail: str = "") -> None:
+        self.events.append(f"{kind} {request.rid}{detail}")
+        if self.on_event is not None:
+            self.on_event(kind, request)
 
     # ---- queue ---------------------------------------------------------------- #
     def add(self, request: Request) -> None:
@@ -112,6 +126,20 @@ class Scheduler:
         room = (reserved + free) * page - self.manager.length(request.rid)
         return max(0, min(wanted, room))
 
+    def _fits_whole(self, request: Request) -> bool:
+        """Whether every group has free pages for the request's known tokens and the headroom
+        (capped by the request's own longest length).  A window group never holds more of a
+        request than its window and one step's tokens."""
+        total = max(len(request), min(len(request) + self.headroom, request.max_len))
+        page = self.manager.page_size
+        for group, free in zip(self.manager.groups, self.manager.free_pages()):
+            need = pages_for(total, page)
+            if group.window is not None:
+                need = min(need, pages_for(group.window - 1 + self.max_tokens_per_step, page) + 1)
+            if need > free:
+                return False
+        return True
+
     def _preempt(self, victim: Request) -> None:
         """Give back a running request's pages; it is recomputed later."""
         self.manager.release(victim.rid)
@@ -121,7 +149,8 @@ class Scheduler:
         victim.preemptions += 1
         self._preempted_now = True
         self.parked.append(victim)
-        self.events.append(f"preempt {victim.rid}")
+        self.n_preemptions += 1
+        self._event("preempt", victim)
 
     def _finish(self, request: Request, reason: str) -> None:
         if request.rid in self.manager:
@@ -131,7 +160,7 @@ class Scheduler:
         request.state = FINISHED
         request.finish_reason = reason
         self.finished.append(request)
-        self.events.append(f"finish {request.rid} {reason}")
+        self._event("finish", request, f" {reason}")
 
     # ---- one step's batch ------------------------------------------------------ #
     def schedule(self) -> List[Scheduled]:
@@ -181,6 +210,8 @@ class Scheduler:
             if not source:
                 break
             request = source[0]
+            if self.running and not self._fits_whole(request):
+                break  # it waits until it fits beside those who run (alone, it takes what there is)
             self.manager.admit(request.rid)
             count = self._tokens_that_fit(request, min(request.pending, budget))
             if count <= 0 or not self.manager.extend(request.rid, count):
@@ -194,7 +225,7 @@ class Scheduler:
             source.popleft()
             request.state = RUNNING
             self.running.append(request)
-            self.events.append(f"admit {request.rid}")
+            self._event("admit", request)
             batch.append(Scheduled(request, request.cached, count, count == request.pending))
             in_batch.add(request.rid)
             budget -= count

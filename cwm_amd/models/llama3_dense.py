@@ -59,6 +59,7 @@ def build_plan(config: Llama3DenseConfig) -> ModelPlan:
         final_norm=norm,
         final_norm_name="norm",
         head_name="output",
+        max_positions=config.max_seq_len,
     )
 
 

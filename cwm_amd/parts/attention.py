@@ -11,6 +11,9 @@ from .base import Mixer, PagedKVSpec, PartChoice, PositionEncoding, Runtime, Ten
 from .linear import LinearWeights
 
 
+MAX_HEAD_DIM = 256  # the attention kernels' largest head size (csrc/attention_simple.hip, attention_mfma.hip)
+
+
 class PagedAttention(Mixer):
     """x -> wo(attention(rope(wq x), cache of rope(wk x), cache of wv x)).
 
@@ -38,6 +41,8 @@ class PagedAttention(Mixer):
     ) -> None:
         if n_heads % n_kv_heads != 0:
             raise ValueError(f"{n_heads} query heads do not divide into {n_kv_heads} key/value heads")
+        if not 1 <= head_dim <= MAX_HEAD_DIM:
+            raise ValueError(f"head_dim {head_dim} is outside 1..{MAX_HEAD_DIM}, the sizes the attention kernels take")
         self.dim = dim
         self.n_heads = n_heads
         self.n_kv_heads = n_kv_heads

@@ -129,7 +129,7 @@ def rope_apply(x: torch.Tensor, positions: torch.Tensor, freqs: torch.Tensor) ->
     re' = re cos - im sin, im' = im cos + re sin; the same rotation for every head.
     x: [T, H, hd]; positions: [T]; freqs: [hd/2].
     """
-    angles = positions.to(torch.float32)[:, None] * freqs.to(torch.float32)[None, :]  # [T, hd/2]
+    angles = positions.to(x.device, torch.float32)[:, None] * freqs.to(x.device, torch.float32)[None, :]  # [T, hd/2]
     cos = torch.cos(angles).to(x.dtype)[:, None, :]
     sin = torch.sin(angles).to(x.dtype)[:, None, :]
     re = x[..., 0::2]
@@ -167,7 +167,7 @@ def attention(
     group = n_q // n_kv
     if scale is None:
         scale = hd ** -0.5
-    pos = torch.arange(n_tok)
+    pos = torch.arange(n_tok, device=q.device)
     distance = pos[:, None] - pos[None, :]  # query position - key position
     allowed = distance >= 0
     if window_left >= 0:
@@ -246,9 +246,10 @@ def forward(
     rnd_h = round_bf16 if rounding == ROUND_AS_REFERENCE else (lambda t: t)
     weights = {name: (t.to(torch.bfloat16) if rounding and t.is_floating_point() else t) for name, t in weights.items()}
     w = {name: t.to(dtype) for name, t in weights.items()}
-    tok = torch.as_tensor(list(tokens), dtype=torch.long)
-    positions = torch.arange(len(tok)) + first_position
-    h = w["tok_embeddings.weight"][tok]
+    table = w["tok_embeddings.weight"]
+    tok = torch.as_tensor(list(tokens), dtype=torch.long, device=table.device)
+    positions = torch.arange(len(tok), device=table.device) + first_position
+    h = table[tok]
     for i in range(n_layers):
         pre = f"layers.{i}."
         x = rnd(rms_norm(h, w[pre + "attention_norm.weight"], norm_eps))

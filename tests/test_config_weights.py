@@ -239,3 +239,15 @@ def test_cli_dotlist(tmp_path):
         load_from_cli(GenerateArgs, ["gen_args.tempreture=1"])
     with pytest.raises(ConfigError, match="key=value"):
         load_from_cli(GenerateArgs, ["--help-me"])
+
+
+def test_a_head_size_no_kernel_takes_is_refused_when_the_model_is_built():
+    """Before any weight is read: a head size above the attention kernels' limit fails as the plan's parts are made."""
+    from cwm_amd.config import parse_config
+    from cwm_amd.models import Model
+
+    data = configs.get("tiny_a")
+    data.update(head_dim=272, dim=64)
+    arch, cfg = parse_config(data)
+    with pytest.raises(ValueError, match="head_dim 272"):
+        Model(arch.build_plan(cfg))

@@ -120,9 +120,10 @@ def test_prompt_logprobs(tmp_path, monkeypatch):
     prompts = {f"p{i}": traces.random_tokens(50 + i, n, vocab) for i, n in enumerate([21, 9, 30])}
     for max_seq in (512, 48):
         engine = _engine(folder, monkeypatch, prompt_logprobs=True, max_prefill=8, max_seq=max_seq, max_batch=3)
+        engine.scheduler.headroom = 0  # requests join as soon as their prompts fit, and outgrow the small cache together
         q = queue.Queue()
         for rid, toks in prompts.items():
-            q.put(Packet(thread_id=rid, tokens=toks, max_gen=6))
+            q.put(Packet(thread_id=rid, tokens=toks, max_gen=12))
         q.put(None)
         out = {p.thread_id: p for p in engine.generate(q) if p is not None}
         if max_seq == 48:
@@ -159,3 +160,62 @@ def test_pool_sizes(tmp_path, monkeypatch):
     assert auto[None] == (int(0.9 * 0.5e9) - auto[8] * per_page_local) // per_page_global
     with pytest.raises(ValueError):
         pool_sizes(model, GenArgs(max_seq=-1), torch.device("cpu"))
+
+
+def _model_without_weights(config):
+    import torch
+    from cwm_amd.config import parse_config
+    from cwm_amd.models import Model
+    from cwm_amd.parts import Runtime
+
+    arch, typed = parse_config(config)
+    model = Model(arch.build_plan(typed))
+    model.runtime = Runtime(torch.device("cpu"), torch.bfloat16)
+    return model
+
+
+CWM_32B_SHAPE = {
+    "architecture": "llama3_dense", "dim": 6144, "n_layers": 64, "n_heads": 48, "n_kv_heads": 8, "head_dim": 128,
+    "vocab_size": 128256, "ffn_dim_multiplier": 1.3125, "multiple_of": 256, "norm_eps": 1e-5, "pos_embed_impl": "scaled_rope",
+    "rope_theta": 1000000.0, "scaled_rope": {"scale_factor": 16, "old_context_len": 8192, "low_freq_factor": 1, "high_freq_factor": 4},
+    "window_attn": {"window_pattern": 4, "local_window": 8192, "global_last_layer": True}, "max_seq_len": 131072,
+}
+
+
+@pytest.mark.parametrize("max_batch", [128, 256])
+def test_default_options_size_the_pools_of_the_32b_shape(max_batch):
+    """max_seq = -1 with the reference's default options at the CWM-32B shape on a 288 GB
+    device: both pools fit into what is free beside 65 GB of weights, neither is reserved for the
+    worst case of max_batch requests, and the split follows the expected request."""
+    import torch
+    from cwm_amd.engine import GenArgs, pool_sizes
+
+    model = _model_without_weights(CWM_32B_SHAPE)
+    free = int(288e9 - 65.2e9)
+    budget = 0.9 * (free - 2e9)
+    page_bytes = 2 * 8 * 128 * 256 * 2  # keys and values of one layer's page of 256 tokens
+    n_global = sum(1 for spec in model.cache_specs if spec.window is None)
+    n_local = len(model.cache_specs) - n_global
+    assert (n_global, n_local) == (17, 47)  # cwm/model/transformer.py:79-85 with pattern 4 and a global last layer
+
+    def bytes_of(sizes):
+        return sizes[None] * n_global * page_bytes + sizes[8192] * n_local * page_bytes
+
+    # the context the configuration names (131,072): a request needs 513 pages of the keep-all
+    # group and 49 of the window group (8,191 + 4,096 tokens)
+    sizes = pool_sizes(model, GenArgs(max_batch=max_batch), torch.device("cuda:0"), free_bytes=free)
+    assert 0.97 * budget <= bytes_of(sizes) <= budget
+    assert abs(sizes[None] / sizes[8192] - 513 / 49) < 0.1
+    assert sizes[None] * 256 >= 8 * 131072  # several requests of full length fit
+    # short requests expected: as many tokens in either group
+    short = pool_sizes(model, GenArgs(max_batch=max_batch, expected_seq=2048), torch.device("cuda:0"), free_bytes=free)
+    assert 0.97 * budget <= bytes_of(short) <= budget
+    assert abs(short[None] - short[8192]) <= 1
+    assert short[8192] < max_batch * 50  # not the worst case of every request
+    # a window group is never larger than max_batch requests can fill; the keep-all group gets the rest
+    few = pool_sizes(model, GenArgs(max_batch=4, expected_seq=2048), torch.device("cuda:0"), free_bytes=free)
+    assert few[8192] == 4 * ((8191 + 4096 + 255) // 256 + 2)
+    assert 0.97 * budget <= bytes_of(few) <= budget
+    # too little memory is an error that says so
+    with pytest.raises(MemoryError, match="no room"):
+        pool_sizes(model, GenArgs(), torch.device("cuda:0"), free_bytes=int(2.1e9))

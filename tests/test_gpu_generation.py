@@ -38,18 +38,87 @@ def test_greedy_generation_float32(tmp_path, name):
     assert again == got
 
 
-def test_temperature_sampling_is_seeded_per_request(tmp_path):
+def _plain_sampled(folder, prompt, n_new, temperature, top_p, stream):
+    """Generation with the plain implementation: softmax(logits / T), the nucleus, and the draw
+    by inverse CDF with the request's own uniform numbers."""
+    from plain import llama3_plain
+
+    config, weights = models.read_folder(folder)
+    toks, out = list(prompt), []
+    for _ in range(n_new):
+        logits = llama3_plain.forward_from_config(weights, config, toks, dtype=torch.float64)[-1]
+        if temperature > 0:
+            probs = llama3_plain.sampling_probabilities(logits, temperature, top_p)
+            nxt = llama3_plain.sample_inverse_cdf(probs, stream.next_uniform())
+        else:
+            nxt = llama3_plain.greedy(logits)
+        toks.append(nxt)
+        out.append(nxt)
+    return out
+
+
+def test_sampled_generation_equals_the_plain_draw(tmp_path):
+    """Prompts of 9, 40 and 100 tokens in portions of 16 beside 24 decode steps at temperature
+    0.7 and top-p 0.9, in float32: every token equals the plain implementation's draw from the
+    plain logits with the request's own stream of uniform numbers, for each request alone and
+    for all in one batch; one request overrides temperature, top-p and seed in its packet,
+    another is greedy by its packet's temperature 0."""
+    import queue
+
+    from cwm_amd.engine import Engine, GenArgs, Packet
+    from cwm_amd.sampling.sampler import RequestStream
+
+    folder = models.make_folder(tmp_path, "tiny_b", seed=8, dtype="float32")
+    vocab = configs.get("tiny_b")["vocab_size"]
+    prompts = {f"p{i}": traces.random_tokens(40 + i, n, vocab) for i, n in enumerate([9, 40, 100, 23])}
+    args = GenArgs(use_sampling=True, temperature=0.7, top_p=0.9, max_batch=4, max_seq=2048, cache_block=16, max_prefill=16,
+                   handover_frequency=3)
+    overrides = {"p1": dict(temperature=1.3, top_p=0.6, seed=777), "p3": dict(temperature=0.0)}
+    engine_seed = 3
+
+    def packet(rid):
+        return Packet(thread_id=rid, tokens=prompts[rid], max_gen=24, **overrides.get(rid, {}))
+
+    want = {}
+    for rid, prompt in prompts.items():
+        o = overrides.get(rid, {})
+        stream = RequestStream(engine_seed, o.get("seed", rid))
+        want[rid] = _plain_sampled(folder, prompt, 24, o.get("temperature", 0.7), o.get("top_p", 0.9), stream)
+    assert want["p0"] != _plain_sampled(folder, prompts["p0"], 24, 0.7, 0.9, RequestStream(engine_seed + 1, "p0"))
+
+    def run(rids):
+        engine = Engine.from_folder(folder, args, dtype="float32", seed=engine_seed)
+        q = queue.Queue()
+        for rid in rids:
+            q.put(packet(rid))
+        q.put(None)
+        out, handovers = {}, 0
+        for pkt in engine.generate(q):
+            if pkt is None:
+                handovers += 1
+            else:
+                out[pkt.thread_id] = pkt.tokens
+        assert handovers == engine.n_steps // 3  # control is handed back every third step
+        return out
+
+    together = run(list(prompts))
+    for rid in prompts:
+        assert together[rid] == want[rid], f"{rid} in a batch: engine {together[rid]} != plain draw {want[rid]}"
+        assert run([rid])[rid] == want[rid], f"{rid} alone"
+
+
+def test_a_request_without_max_gen_runs_until_the_cache_is_full(tmp_path):
+    """max_gen None in the options and in the packet: the request's longest length is the cache's
+    (cwm/fastgen/generate.py:91-96), and it ends with reason "length" there."""
     from cwm_amd.engine import Engine, GenArgs
 
-    folder = models.make_folder(tmp_path, "tiny_b", seed=8, dtype="bfloat16")
-    vocab = configs.get("tiny_b")["vocab_size"]
-    prompts = [traces.random_tokens(40 + i, n, vocab) for i, n in enumerate([9, 40, 100])]
-    args = GenArgs(use_sampling=True, temperature=0.7, top_p=0.9, max_batch=4, max_seq=2048, cache_block=16, max_prefill=16)
-    a = Engine.from_folder(folder, args, dtype="bfloat16", seed=3).generate_tokens(prompts, max_gen=24)
-    b = Engine.from_folder(folder, args, dtype="bfloat16", seed=3).generate_tokens(prompts, max_gen=24)
-    c = Engine.from_folder(folder, args, dtype="bfloat16", seed=4).generate_tokens(prompts, max_gen=24)
-    assert a == b and a != c
-    assert all(len(x) == 24 for x in a)
+    folder = models.make_folder(tmp_path, "tiny_a", seed=8, dtype="float32")
+    vocab = configs.get("tiny_a")["vocab_size"]
+    prompt = traces.random_tokens(5, 10, vocab)
+    engine = Engine.from_folder(folder, GenArgs(use_sampling=False, max_batch=2, max_seq=64, cache_block=16, max_gen=None), dtype="float32")
+    got = engine.generate_tokens([prompt])[0]
+    assert len(prompt) + len(got) == 64
+    assert got == generation.plain_greedy(folder, prompt, 54)
 
 
 def test_command_line_child_process(tmp_path):
@@ -205,6 +274,22 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
             torch.testing.assert_close(cut[k], whole[k], rtol=1e-4, atol=1e-5)
         # the state matters: another request's logits differ from a fresh run of the same tokens after other input
         assert not torch.allclose(whole["a"][5], whole["a"][4])
+
+        # a state slot that is used again starts at zero: with one slot, "b" after "a" gives what "b" alone gives
+        manager = CacheManager(model.cache_specs, 4, 64, 1)
+        storage = CacheStorage(manager, runtime.device, runtime.act_dtype)
+        runner = ModelRunner(model, manager, storage)
+        toks_a, toks_b = traces.random_tokens(1, 23, 61), traces.random_tokens(2, 17, 61)
+        slot_a = runner.admit("a")
+        assert manager.extend("a", 23)
+        runner.step([Portion("a", toks_a, [22])])
+        assert all(float(t[slot_a].abs().max()) > 0 for t in storage.state.values())  # it has left its sums there
+        runner.release("a")
+        slot_b = runner.admit("b")
+        assert slot_b == slot_a
+        assert manager.extend("b", 17)
+        after = runner.step([Portion("b", toks_b, list(range(17)))]).cpu()
+        torch.testing.assert_close(after, whole["b"], rtol=1e-4, atol=1e-5)
     finally:
         del MIXERS["toy_running_sum"]
         del ARCHITECTURES["toy_state_model"]

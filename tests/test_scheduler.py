@@ -18,10 +18,10 @@ def next_token(tokens):
     return acc % VOCAB
 
 
-def run(prompts, num_pages, page_size=4, max_batch=4, budget=16, max_gen=12, stop=(), window=None, trace=None):
+def run(prompts, num_pages, page_size=4, max_batch=4, budget=16, max_gen=12, stop=(), window=None, trace=None, headroom=0):
     specs = [PagedKVSpec(1, 8, None), PagedKVSpec(1, 8, window)]
     manager = CacheManager(specs, page_size, num_pages, max_batch)
-    sched = Scheduler(manager, max_batch, budget)
+    sched = Scheduler(manager, max_batch, budget, headroom=headroom)
     for i, p in enumerate(prompts):
         sched.add(Request(rid=i, prompt=list(p), max_len=len(p) + max_gen))
     steps = 0
@@ -132,6 +132,55 @@ def test_window_group_lets_longer_sequences_fit():
     # 8 pages of 4 tokens hold 32 tokens; the windowed group frees pages as it goes, the keep-all group is the limit
     done, _ = run([[1] * 10], num_pages=8, page_size=4, max_gen=20, window=6)
     assert done[0].finish_reason == "length" and len(done[0].generated) == 20
+
+
+def test_no_admission_and_preemption_in_turns_under_page_pressure():
+    """Two requests that cannot both grow to their full length in the pool: the second is let in
+    only when its known tokens fit beside the first, is preempted at most once when both outgrow
+    the pool, and then waits until it fits again, instead of being admitted with a part of its
+    prompt, losing it as the shortest request, and coming back every other step."""
+    prompts = [[1] * 18, [2] * 18]
+    trace = []
+    done, sched = run(prompts, num_pages=10, page_size=4, max_batch=4, budget=16, max_gen=22, trace=trace)
+    for i, p in enumerate(prompts):
+        assert done[i].generated == expected(p, 22)
+    assert sched.n_preemptions <= 1
+    scheduled = sum(c for step in trace for _, c in step)
+    needed = sum(len(p) + 22 - 1 for p in prompts)  # every token but the last generated one runs once
+    assert scheduled <= needed + 18 + 22  # at most one request is computed twice
+    # with room to decode asked for at admission there is no preemption at all: the second waits
+    done, sched = run(prompts, num_pages=10, page_size=4, max_batch=4, budget=16, max_gen=22, headroom=22)
+    assert sched.n_preemptions == 0
+    for i, p in enumerate(prompts):
+        assert done[i].generated == expected(p, 22)
+
+
+def test_a_request_joins_others_only_when_it_fits_whole():
+    sched_trace = []
+    # 12 pages of 4: the first request holds 10 after its prompt; the second's 12 tokens need 3
+    done, sched = run([[1] * 40, [2] * 12], num_pages=12, page_size=4, budget=64, max_gen=4, trace=sched_trace)
+    events = list(sched.events)
+    assert events.index("admit 1") > events.index("finish 0 length")
+    assert sched.n_preemptions == 0
+    # a shorter first request leaves room for it at once
+    done, sched = run([[1] * 30, [2] * 12], num_pages=12, page_size=4, budget=64, max_gen=4)
+    events = list(sched.events)
+    assert events.index("admit 1") < events.index("finish 0 length")
+
+
+def test_events_and_finished_requests_do_not_pile_up():
+    manager = CacheManager([PagedKVSpec(1, 8, None)], 4, 64, 2)
+    sched = Scheduler(manager, 2, 8)
+    assert sched.events.maxlen is not None
+    seen = []
+    sched.on_event = lambda kind, request: seen.append((kind, request.rid))
+    sched.add(Request(rid="x", prompt=[1, 2, 3], max_len=4))
+    batch = sched.schedule()
+    for item in batch:
+        manager.advance(item.request.rid, item.count)
+    sched.step_done(batch, [5], set())
+    assert seen == [("admit", "x"), ("finish", "x")]
+    assert [r.rid for r in sched.finished] == ["x"]
 
 
 def test_empty_prompt_is_refused():
