@@ -219,3 +219,42 @@ def test_default_options_size_the_pools_of_the_32b_shape(max_batch):
     # too little memory is an error that says so
     with pytest.raises(MemoryError, match="no room"):
         pool_sizes(model, GenArgs(), torch.device("cuda:0"), free_bytes=int(2.1e9))
+
+
+def test_metrics_log_and_profile_window(tmp_path, monkeypatch):
+    """FG_METRICS names a file that receives the scheduler's events as JSON lines (the
+    reference's kinds `nactive`, `yield`, `unpark`, and `preempt`); request_profile() traces
+    the next FG_PROFILE_ITERS steps and leaves a Chrome trace in FG_PROFILE_DIR."""
+    import gzip
+
+    path = tmp_path / "metrics.jsonl"
+    monkeypatch.setenv("FG_METRICS", str(path))
+    monkeypatch.setenv("FG_PROFILE_ITERS", "2")
+    monkeypatch.setenv("FG_PROFILE_DIR", str(tmp_path))
+    folder = models.make_folder(tmp_path, "tiny_a", seed=2, dtype="float32")
+    vocab = configs.get("tiny_a")["vocab_size"]
+    prompts = [traces.random_tokens(10 + i, n, vocab) for i, n in enumerate([12, 25, 7, 18])]
+    engine = _engine(folder, monkeypatch, max_seq=64)
+    engine.scheduler.headroom = 0
+    engine.request_profile()
+    got = engine.generate_tokens(prompts, max_gen=12)
+    engine.metrics.close()
+    records = [json.loads(line) for line in path.read_text().splitlines()]
+    kinds = [r["kind"] for r in records]
+    assert kinds.count("yield") == len(prompts)
+    assert sorted(r["tokens"] for r in records if r["kind"] == "yield") == sorted(len(g) for g in got)
+    assert "nactive" in kinds and all("timestamp" in r for r in records)
+    first = next(r for r in records if r["kind"] == "nactive")
+    assert first["lanes"] >= 1 and len(first["free_pages"]) == len(engine.manager.groups)
+    assert kinds.count("preempt") == engine.scheduler.n_preemptions >= 1
+    assert kinds.count("unpark") >= 1
+    # the trace of two steps
+    assert engine.last_profile_path is not None and engine.last_profile_path.startswith(str(tmp_path))
+    with gzip.open(engine.last_profile_path, "rt") as fh:
+        trace = json.load(fh)
+    assert trace["traceEvents"]
+    # without the variable nothing is written
+    monkeypatch.delenv("FG_METRICS")
+    other = _engine(folder, monkeypatch)
+    other.generate_tokens(prompts[:1], max_gen=2)
+    assert len(path.read_text().splitlines()) == len(records)

@@ -194,6 +194,157 @@ def test_one_head_no_rotation_is_library_attention():
     torch.testing.assert_close(plain.attention(q, k, v), want)
 
 
+# ---- the composition of a layer and of the model ------------------------------------------------- #
+_CFG = dict(dim=32, n_layers=1, n_heads=4, n_kv_heads=2, head_dim=8, hidden=48, vocab_size=50)
+
+
+def _kw(n_layers=1, window_left=None, theta=100.0):
+    return dict(n_layers=n_layers, n_heads=4, n_kv_heads=2, head_dim=8, norm_eps=1e-5, rope_freqs=plain.rope_frequencies(8, theta),
+                window_left=window_left or [-1] * n_layers, dtype=torch.float64)
+
+
+def test_one_layer_composed_from_library_routines():
+    """A one-layer model put together here from F.rms_norm, F.linear, a complex product for the
+    rotation, F.scaled_dot_product_attention and F.silu, in the order of
+    cwm/fastgen/forward.py:563-821, equals `forward`: the place of each norm, of the residual
+    sums, of the final norm and the head."""
+    w = {k: v.double() for k, v in _tiny_weights(_CFG, seed=3).items()}
+    toks = [3, 7, 1, 9, 30, 2, 11]
+    d, hq, hkv, hd = 32, 4, 2, 8
+    h = w["tok_embeddings.weight"][toks]
+    x = F.rms_norm(h, (d,), w["layers.0.attention_norm.weight"], 1e-5)
+    q = F.linear(x, w["layers.0.attention.wq.weight"]).view(-1, hq, hd)
+    k = F.linear(x, w["layers.0.attention.wk.weight"]).view(-1, hkv, hd)
+    v = F.linear(x, w["layers.0.attention.wv.weight"]).view(-1, hkv, hd)
+    angles = torch.arange(len(toks)).double()[:, None] * plain.rope_frequencies(hd, 100.0).double()[None, :]
+    turn = torch.polar(torch.ones_like(angles), angles)[:, None, :]
+    q = torch.view_as_real(torch.view_as_complex(q.reshape(-1, hq, hd // 2, 2)) * turn).reshape(-1, hq, hd)
+    k = torch.view_as_real(torch.view_as_complex(k.reshape(-1, hkv, hd // 2, 2)) * turn).reshape(-1, hkv, hd)
+    att = F.scaled_dot_product_attention(
+        q.transpose(0, 1), k.repeat_interleave(hq // hkv, dim=1).transpose(0, 1), v.repeat_interleave(hq // hkv, dim=1).transpose(0, 1), is_causal=True
+    ).transpose(0, 1)
+    h = h + F.linear(att.reshape(len(toks), -1), w["layers.0.attention.wo.weight"])
+    x = F.rms_norm(h, (d,), w["layers.0.ffn_norm.weight"], 1e-5)
+    h = h + F.linear(F.silu(F.linear(x, w["layers.0.feed_forward.w1.weight"])) * F.linear(x, w["layers.0.feed_forward.w3.weight"]),
+                     w["layers.0.feed_forward.w2.weight"])
+    want = F.linear(F.rms_norm(h, (d,), w["norm.weight"], 1e-5), w["output.weight"])
+    torch.testing.assert_close(plain.forward(w, toks, **_kw()), want, rtol=1e-6, atol=1e-8)
+
+
+def test_layers_that_add_nothing_leave_head_of_norm_of_embedding():
+    """wo = w2 = 0: both updates vanish and the logits are head(norm(embedding)); with only
+    w2 = 0 they are not (the attention's update is added to the stream, not lost)."""
+    w = {k: v.double() for k, v in _tiny_weights(dict(_CFG, n_layers=2), seed=4).items()}
+    toks = [5, 9, 2, 40]
+    for i in range(2):
+        w[f"layers.{i}.feed_forward.w2.weight"] = torch.zeros_like(w[f"layers.{i}.feed_forward.w2.weight"])
+    with_attention = plain.forward(w, toks, **_kw(2))
+    for i in range(2):
+        w[f"layers.{i}.attention.wo.weight"] = torch.zeros_like(w[f"layers.{i}.attention.wo.weight"])
+    want = F.linear(F.rms_norm(w["tok_embeddings.weight"][toks], (32,), w["norm.weight"], 1e-5), w["output.weight"])
+    torch.testing.assert_close(plain.forward(w, toks, **_kw(2)), want)
+    assert not torch.allclose(with_attention, want)
+
+
+def test_pre_norm_makes_the_attention_update_blind_to_the_streams_scale():
+    """The attention reads the normalised stream: with the embedding scaled by c (and eps tiny) its
+    update u stays what it was, so the stream after it is c * e + u.  (A norm after the sum, or none,
+    would scale u with c.)  The feed-forward adds nothing here (w2 = 0); the stream is read off
+    through an identity head behind the final norm, which keeps its direction: the two
+    directions n_c for c = 1 and c = 3 must satisfy r3 * n_3 - r1 * n_1 = 2 e for some lengths."""
+    cfg = dict(_CFG, vocab_size=32)
+    w = {k: v.double() for k, v in _tiny_weights(cfg, seed=5).items()}
+    w["output.weight"] = torch.eye(32, dtype=torch.float64)
+    w["norm.weight"] = torch.ones(32, dtype=torch.float64)
+    w["layers.0.feed_forward.w2.weight"] = torch.zeros_like(w["layers.0.feed_forward.w2.weight"])
+    toks = [5, 9, 2, 31, 7]
+    emb = w["tok_embeddings.weight"][toks]
+    kw = _kw()
+    kw["norm_eps"] = 1e-30
+
+    def direction(c):
+        return plain.forward(dict(w, **{"tok_embeddings.weight": c * w["tok_embeddings.weight"]}), toks, **kw)
+
+    n1, n3 = direction(1.0), direction(3.0)
+    for row in range(len(toks)):
+        a = torch.stack([n3[row], -n1[row]], dim=1)  # [32, 2], unknown lengths (r3, r1)
+        rhs = (2 * emb[row]).unsqueeze(1)
+        sol = torch.linalg.lstsq(a, rhs).solution
+        assert float((a @ sol - rhs).abs().max()) < 1e-9 and float(sol.min()) > 0
+    # and the update is not nothing: the stream is not parallel to the embedding
+    assert not torch.allclose(n1, F.rms_norm(emb, (32,), None, 1e-30))
+
+
+def test_projection_rows_belong_to_heads_in_blocks():
+    """Output feature f of wq, wk, wv belongs to head f // head_dim (the views of
+    cwm/fastgen/forward.py:606-608).  With the rows of one query head zero, that head's scores
+    are all equal and it returns the running mean of its key/value head's values; with wo zero
+    outside that head's columns nothing else reaches the stream."""
+    w = {k: v.double() for k, v in _tiny_weights(_CFG, seed=6).items()}
+    d, hq, hkv, hd = 32, 4, 2, 8
+    head = 2  # reads key/value head 1
+    w["layers.0.attention.wq.weight"][head * hd : (head + 1) * hd] = 0
+    wo = torch.zeros_like(w["layers.0.attention.wo.weight"])
+    wo[:, head * hd : (head + 1) * hd] = w["layers.0.attention.wo.weight"][:, head * hd : (head + 1) * hd]
+    w["layers.0.attention.wo.weight"] = wo
+    w["layers.0.feed_forward.w2.weight"] = torch.zeros_like(w["layers.0.feed_forward.w2.weight"])
+    w["output.weight"] = torch.eye(32, dtype=torch.float64)
+    w["norm.weight"] = torch.ones(32, dtype=torch.float64)
+    w = dict(w, **{"tok_embeddings.weight": w["tok_embeddings.weight"][:32]})
+    toks = [5, 9, 2, 31, 7, 7]
+    emb = w["tok_embeddings.weight"][toks]
+    x = F.rms_norm(emb, (d,), w["layers.0.attention_norm.weight"], 1e-5)
+    v = F.linear(x, w["layers.0.attention.wv.weight"])[:, (head // 2) * hd : (head // 2 + 1) * hd]  # key/value head 1
+    running_mean = torch.cumsum(v, 0) / torch.arange(1, len(toks) + 1).double()[:, None]
+    stream = emb + running_mean @ wo[:, head * hd : (head + 1) * hd].T
+    torch.testing.assert_close(plain.forward(w, toks, **_kw()), F.rms_norm(stream, (d,), None, 1e-5))
+
+
+def test_window_of_w_keys_reaches_w_minus_one_back_per_layer():
+    """local_window = W means W keys, the query's own included (window_left = W - 1,
+    cwm/model/transformer.py:253-270): through two layers with W = 2 the logits at a position
+    depend on the two tokens before it and on nothing earlier; with W = 1 on the token alone."""
+    w = {k: v.double() for k, v in _tiny_weights(dict(_CFG, n_layers=2), seed=7).items()}
+    cfg = dict(dim=32, n_layers=2, n_heads=4, n_kv_heads=2, head_dim=8, vocab_size=50, rope_theta=100.0,
+               window_attn={"window_pattern": 2, "local_window": 2, "global_window": 2, "global_last_layer": True})
+    toks = [3, 7, 1, 9, 30, 2, 11]
+    base = plain.forward_from_config(w, cfg, toks, dtype=torch.float64)
+    far = plain.forward_from_config(w, cfg, toks[:3] + [44] + toks[4:], dtype=torch.float64)  # position 3 changes
+    torch.testing.assert_close(far[6], base[6])  # three back: out of reach of position 6
+    assert not torch.allclose(far[5], base[5])  # two back: within reach of position 5
+    cfg["window_attn"].update(local_window=1, global_window=1)
+    alone = plain.forward_from_config(w, cfg, toks, dtype=torch.float64)
+    other = plain.forward_from_config(w, cfg, [8, 8, 8, 8, 8, 8, 11], dtype=torch.float64)
+    torch.testing.assert_close(alone[6], other[6])
+    # explicit layer kinds name their windows: a "local" layer takes local_window, a "global" one global_window
+    cfg["window_attn"].update(local_window=2, global_window=None)
+    cfg["layer_types"] = ["global", "local"]
+    mixed = plain.forward_from_config(w, cfg, toks, dtype=torch.float64)
+    assert not torch.allclose(plain.forward_from_config(w, cfg, [44] + toks[1:], dtype=torch.float64)[6], mixed[6])  # layer 0 sees all
+
+
+def test_bfloat16_emulation_rounds_where_it_says():
+    """Both emulations differ from the exact run on the same (bfloat16) weights by a few of
+    bfloat16's relative steps; the reference's bfloat16 stream costs more than the engine's
+    float32 stream; only the reference rounds its logits; probabilities are rounded in both."""
+    cfg = dict(dim=32, n_layers=3, n_heads=4, n_kv_heads=2, head_dim=8, hidden=48, vocab_size=50)
+    w = _tiny_weights(cfg, seed=8)
+    toks = list(range(3, 40))
+    kw = _kw(3)
+    exact = plain.forward({k: v.bfloat16() for k, v in w.items()}, toks, **kw)
+    eng = plain.forward(w, toks, rounding=plain.ROUND_AS_ENGINE, **kw)
+    ref = plain.forward(w, toks, rounding=plain.ROUND_AS_REFERENCE, **kw)
+    scale = exact.abs().max()
+    e_eng, e_ref = (eng - exact).abs().max() / scale, (ref - exact).abs().max() / scale
+    assert 1e-4 < e_eng < 3e-2 and 1e-4 < e_ref < 5e-2
+    assert ((ref - exact) ** 2).mean() > ((eng - exact) ** 2).mean()
+    assert torch.equal(ref, plain.round_bf16(ref)) and not torch.equal(eng, plain.round_bf16(eng))  # only the reference rounds its logits
+    q = torch.randn(9, 2, 8, dtype=torch.float64)
+    assert not torch.equal(plain.attention(q, q, q, round_probabilities=True), plain.attention(q, q, q))
+    with pytest.raises(ValueError):
+        plain.forward(w, toks, rounding="half", **kw)
+
+
 # ---- sampling ------------------------------------------------------------------------------ #
 def test_sampling_probabilities():
     logits = torch.randn(40)
