@@ -8,10 +8,11 @@
 
 CWM_DEFINE_ERROR_API
 
-// ---- embedding: out[t, :] = table[token[t], :] as float32 --------------------- //
+// ---- embedding: out[t, :] = scale * table[token[t], :] as float32 -------------- //
+// (scale is 1 for the architecture of the reference; others multiply the embedding)
 template <typename TW>
 __global__ void embedding_kernel(float* __restrict__ out, const TW* __restrict__ table,
-                                 const int* __restrict__ tokens, int dim, int vocab) {
+                                 const int* __restrict__ tokens, int dim, int vocab, float scale) {
   const int t = blockIdx.x;
   const int tok = tokens[t];
   float* dst = out + (size_t)t * dim;
@@ -20,20 +21,20 @@ __global__ void embedding_kernel(float* __restrict__ out, const TW* __restrict__
     return;
   }
   const TW* src = table + (size_t)tok * dim;
-  for (int i = threadIdx.x; i < dim; i += blockDim.x) dst[i] = Elem<TW>::load(src + i);
+  for (int i = threadIdx.x; i < dim; i += blockDim.x) dst[i] = scale * Elem<TW>::load(src + i);
 }
 
 extern "C" int cwm_embedding(void* out, const void* table, int table_dtype, const int* tokens,
-                             int n_tokens, int dim, int vocab, hipStream_t stream) {
+                             int n_tokens, int dim, int vocab, float scale, hipStream_t stream) {
   CWM_REQUIRE(n_tokens >= 0 && dim > 0 && vocab > 0, "embedding: bad sizes T=%d D=%d V=%d", n_tokens, dim, vocab);
   if (n_tokens == 0) return 0;
   const int threads = dim >= 1024 ? 256 : (dim >= 256 ? 128 : 64);
   if (table_dtype == CWM_F32)
     hipLaunchKernelGGL(embedding_kernel<float>, dim3(n_tokens), dim3(threads), 0, stream, (float*)out,
-                       (const float*)table, tokens, dim, vocab);
+                       (const float*)table, tokens, dim, vocab, scale);
   else if (table_dtype == CWM_BF16)
     hipLaunchKernelGGL(embedding_kernel<bf16_t>, dim3(n_tokens), dim3(threads), 0, stream, (float*)out,
-                       (const bf16_t*)table, tokens, dim, vocab);
+                       (const bf16_t*)table, tokens, dim, vocab, scale);
   else
     return cwm_fail("embedding: unknown table dtype %d", table_dtype);
   return cwm_launch_status("embedding");

@@ -32,13 +32,16 @@ def parse_dtype(dtype: Union[str, torch.dtype]) -> torch.dtype:
         raise ValueError(f"dtype must be one of {', '.join(_DTYPES)}, found {dtype!r}") from None
 
 
-def load_model(folder: str, dtype: Union[str, torch.dtype], device: Union[str, torch.device]) -> Tuple[Model, Any]:
-    """The model that `folder/config.json` names, with the folder's tensors."""
+def load_model(
+    folder: str, dtype: Union[str, torch.dtype], device: Union[str, torch.device], keep_float32: bool = False
+) -> Tuple[Model, Any]:
+    """The model that `folder/config.json` names, with the folder's tensors.  In bfloat16 mode
+    matrices stored in 32 bits are cast to bfloat16 unless `keep_float32`."""
     device = torch.device(device)
     act_dtype = parse_dtype(dtype)
     arch, config = load_config(folder)
     model = Model(arch.build_plan(config))
-    tensors = load_tensors(folder, model.tensor_specs(), act_dtype, device)
+    tensors = load_tensors(folder, model.tensor_specs(), act_dtype, device, keep_float32)
     model.bind(tensors, Runtime(device=device, act_dtype=act_dtype))
     return model, config
 

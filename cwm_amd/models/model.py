@@ -25,7 +25,7 @@ class Model:
                 BLOCKS[layer.block](
                     norm1=layer.norm.build("norm"),
                     mixer=layer.mixer.build("mixer"),
-                    norm2=layer.norm.build("norm"),
+                    norm2=(layer.norm2 or layer.norm).build("norm"),
                     feed_forward=layer.feed_forward.build("feed_forward"),
                     names=layer.names,
                 )
@@ -62,10 +62,9 @@ class Model:
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         """Every tensor of the model folder by its full name."""
         plan = self.plan
-        specs: Dict[str, TensorSpec] = {
-            plan.embedding_name + ".weight": TensorSpec((plan.vocab_size, plan.dim)),
-            plan.head_name + ".weight": TensorSpec((plan.vocab_size, plan.dim)),
-        }
+        specs: Dict[str, TensorSpec] = {plan.embedding_name + ".weight": TensorSpec((plan.vocab_size, plan.dim))}
+        if not plan.tied_head:
+            specs[plan.head_name + ".weight"] = TensorSpec((plan.vocab_size, plan.dim))
         for layer, block in zip(plan.layers, self.blocks):
             for name, spec in block.tensor_specs().items():
                 specs[layer.prefix + name] = spec
@@ -77,7 +76,7 @@ class Model:
         plan = self.plan
         self.runtime = runtime
         self.embedding = tensors[plan.embedding_name + ".weight"].contiguous()
-        self.head = LinearWeights(tensors[plan.head_name + ".weight"])
+        self.head = LinearWeights(self.embedding if plan.tied_head else tensors[plan.head_name + ".weight"])
         for layer, block in zip(plan.layers, self.blocks):
             prefix = layer.prefix
             block.bind({n[len(prefix):]: t for n, t in tensors.items() if n.startswith(prefix)}, runtime)
@@ -92,7 +91,7 @@ class Model:
         Order as cwm/fastgen/forward.py:543-821: embedding, layers, final norm on
         the wanted rows, output projection, float32 logits.
         """
-        h = ops.embedding(batch.tokens, self.embedding)
+        h = ops.embedding(batch.tokens, self.embedding, 1.0 if self.plan.embedding_scale is None else self.plan.embedding_scale)
         delta = None
         for call, slot, writes in zip(self.run_order, self.cache_slot, self.writes_cache):
             view = cache.view(slot, batch)

@@ -74,31 +74,59 @@ class PagedAttention(Mixer):
 
     def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
         super().bind(tensors, runtime)
-        names = ("wq", "wk", "wv")
-        self.qkv = LinearWeights.joined(
-            [tensors[f"{n}.weight"] for n in names],
-            [tensors.get(f"{n}.bias") for n in names],
-        )
-        self.wo = LinearWeights(tensors["wo.weight"])
         if self.position_encoding is not None:
             self.position_encoding.bind({}, runtime)
+        names = ("wq", "wk", "wv")
+        weights = {n: tensors[f"{n}.weight"] for n in names}
+        biases = {n: tensors.get(f"{n}.bias") for n in names}
+        pairing = self.position_encoding.rotary_pairing() if self.position_encoding is not None else "adjacent"
+        if pairing == "halves":
+            # the kernels turn adjacent elements: bring element i and i + head_dim / 2 of every query and key
+            # head side by side, once, by the order of the projections' rows
+            half = self.head_dim // 2
+            order = torch.stack([torch.arange(half), torch.arange(half) + half], dim=1).reshape(-1)
+            for n, heads in (("wq", self.n_heads), ("wk", self.n_kv_heads)):
+                rows = (torch.arange(heads)[:, None] * self.head_dim + order[None, :]).reshape(-1).to(weights[n].device)
+                weights[n] = weights[n][rows]
+                if biases[n] is not None:
+                    biases[n] = biases[n][rows]
+        elif pairing != "adjacent":
+            raise ValueError(f"rotary pairing {pairing!r}: 'adjacent' and 'halves' are known")
+        self.qkv = LinearWeights.joined([weights[n] for n in names], [biases[n] for n in names])
+        self.wo = LinearWeights(tensors["wo.weight"])
+        # a subclass that changes queries and keys between projection and rotation cannot use the fused product
+        self._plain_projection = type(self).transform_qk is not PagedAttention.transform_qk
+
+    def transform_qk(self, q: torch.Tensor, k: Optional[torch.Tensor], batch: Any) -> None:
+        """The seam between projection and rotation: a subclass may change the projected queries
+        `q` [T, Hq, hd] and keys `k` [T, Hkv, hd] (None when this call writes no cache) in place
+        here (a norm per head, say) before they are rotated and the keys are cached.  Overriding it
+        takes the step off the fused projection + rotation + cache-write kernel."""
 
     def forward(self, x: torch.Tensor, batch: Any, cache: Any, write_cache: bool = True) -> torch.Tensor:
         hd = self.head_dim
         q_out = self.n_heads * hd
+        kv_out = self.n_kv_heads * hd
         table = self.position_encoding.rotary_table() if self.position_encoding is not None else None
-        if write_cache:
+        if write_cache and not self._plain_projection:
             qkv = ops.qkv_rope_write(
                 x, self.qkv.weight, self.qkv.bias, self.n_heads, self.n_kv_heads, hd,
                 batch.positions, table, cache.cache, cache.block_table, batch.seq_of_token,
             )
             q = qkv[:, :q_out].unflatten(1, (self.n_heads, hd))
         else:
-            # reads a cache that another layer wrote in this step: only the queries are needed
             qkv = self.qkv(x)
             q = qkv[:, :q_out].unflatten(1, (self.n_heads, hd))
-            if table is not None:
-                ops.rope_kv_write(q, None, None, batch.positions, table)
+            if write_cache:
+                k = qkv[:, q_out : q_out + kv_out].unflatten(1, (self.n_kv_heads, hd))
+                v = qkv[:, q_out + kv_out :].unflatten(1, (self.n_kv_heads, hd))
+                self.transform_qk(q, k, batch)
+                ops.rope_kv_write(q, k, v, batch.positions, table, cache.cache, cache.block_table, batch.seq_of_token)
+            else:
+                # reads a cache that another layer wrote in this step: only the queries are needed
+                self.transform_qk(q, None, batch)
+                if table is not None:
+                    ops.rope_kv_write(q, None, None, batch.positions, table)
         attn = ops.paged_attention(q, cache.cache, cache.block_table, batch, self.window, self.scale)
         return self.wo(attn, partials_ok=True)  # added into the residual by the next norm
 

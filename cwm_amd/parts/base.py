@@ -29,6 +29,11 @@ class TensorSpec:
     shape: Tuple[int, ...]
     kind: str = "float"  # "float" or "int" (integer tables are kept as int32)
     init: str = "normal"  # how the random-weights writer fills it: "normal" | "norm" | "zeros"
+    # type a floating tensor is kept in when the model runs in bfloat16: "activation" casts it to
+    # bfloat16 whatever it is stored in (matrices: every product then runs on the bfloat16 kernels, as the
+    # reference casts every parameter, cwm/model/parallelize_transformer.py:50-59); "stored" keeps a
+    # tensor that is stored in 32 bits in float32 (norm weights, tables whose precision matters)
+    precision: str = "activation"
 
 
 # --------------------------------------------------------------------------- #
@@ -104,6 +109,14 @@ class PositionEncoding(Part):
 
     def rotary_table(self) -> Optional[torch.Tensor]:
         return None
+
+    def rotary_pairing(self) -> str:
+        """Which two elements of a head the i-th frequency turns: "adjacent" (2i, 2i + 1), the
+        reference's (cwm/fastgen/kernels/rope.py:71-87), or "halves" (i, i + head_dim / 2).  The
+        kernels turn adjacent pairs; a mixer serves "halves" by reordering, once at load time, the
+        rows of its query and key projections so that each pair lies side by side (scores are sums
+        over a head's elements, so a common reordering of queries and keys changes nothing else)."""
+        return "adjacent"
 
 
 class Mixer(Part):
@@ -195,7 +208,8 @@ class LayerPlan:
         BLOCKS[block](norm1=Norm, mixer=Mixer, norm2=Norm, feed_forward=FeedForward, names=names)
     where `names` maps each of these four roles to the prefix of its tensors below
     `prefix` (for instance {"norm1": "attention_norm.", "mixer": "attention.", ...}).
-    A position encoding is an argument of the mixer that applies it.
+    `norm` is the norm before the mixer and, unless `norm2` names another, also the one
+    before the feed-forward.  A position encoding is an argument of the mixer that applies it.
     """
 
     prefix: str
@@ -204,6 +218,7 @@ class LayerPlan:
     mixer: PartChoice
     feed_forward: PartChoice
     names: Mapping[str, str]
+    norm2: Optional[PartChoice] = None
 
 
 @dataclass(frozen=True)
@@ -225,5 +240,7 @@ class ModelPlan:
     run_order: List[LayerCall]
     final_norm: PartChoice
     final_norm_name: str
-    head_name: str
-    max_positions: Optional[int] = None
+    head_name: str  # ignored with `tied_head`
+    max_positions: Optional[int] = None  # the context length the configuration names (cache sizing reads it)
+    embedding_scale: Optional[float] = None  # the embedding is multiplied by it (None: as it is)
+    tied_head: bool = False  # the output projection is the embedding table; the folder holds no head tensor

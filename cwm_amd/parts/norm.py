@@ -21,7 +21,7 @@ class RMSNorm(Norm):
         self.eps = float(eps)
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {"weight": TensorSpec((self.dim,), init="norm")}
+        return {"weight": TensorSpec((self.dim,), init="norm", precision="stored")}
 
     def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
         super().bind(tensors, runtime)

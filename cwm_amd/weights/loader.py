@@ -7,8 +7,12 @@ cwm/fastgen/utils/loading.py:57-60), and casts every parameter to bfloat16
 lists every missing tensor, every unexpected one and every wrong shape.
 
 Storage types after loading:
-  activation type bfloat16: tensors stored in 16 bits become bfloat16, tensors
-    stored in 32 (or 64) bits stay float32, integer tables become int32;
+  activation type bfloat16: tensors stored in 16 bits become bfloat16; a tensor stored
+    in 32 (or 64) bits becomes bfloat16 too if its spec has precision "activation"
+    (the matrices: the reference casts every parameter,
+    cwm/model/parallelize_transformer.py:50-59, and the bfloat16 kernels need them so)
+    and stays float32 if its spec says "stored" (norm weights) or the caller asks to
+    keep 32-bit tensors as they are; integer tables become int32;
   activation type float32: every floating tensor becomes float32.
 """
 
@@ -39,13 +43,17 @@ def weight_files(folder: str) -> List[str]:
     return files
 
 
-def target_dtype(stored: str, kind: str, act_dtype: torch.dtype, name: str) -> torch.dtype:
-    """Type a tensor is kept in, from how it is stored."""
+def target_dtype(
+    stored: str, kind: str, act_dtype: torch.dtype, name: str, precision: str = "activation", keep_float32: bool = False
+) -> torch.dtype:
+    """Type a tensor is kept in, from how it is stored and what its spec asks."""
     if kind == "int":
         if stored not in _INTS:
             raise WeightError(f"{name}: an integer table is stored as {stored}")
         return torch.int32
     if stored in _FLOAT_WIDE:
+        if act_dtype == torch.bfloat16 and precision == "activation" and not keep_float32:
+            return torch.bfloat16
         return torch.float32
     if stored in _FLOAT_16:
         return torch.float32 if act_dtype == torch.float32 else torch.bfloat16
@@ -57,8 +65,11 @@ def load_tensors(
     specs: Mapping[str, TensorSpec],
     act_dtype: torch.dtype,
     device: torch.device,
+    keep_float32: bool = False,
 ) -> Dict[str, torch.Tensor]:
-    """All tensors that `specs` names, checked and moved to `device`."""
+    """All tensors that `specs` names, checked and moved to `device`.  `keep_float32`: in
+    bfloat16 mode, tensors stored in 32 bits all stay float32 (their products then run on the
+    float32 kernel)."""
     from safetensors import safe_open
 
     where: Dict[str, str] = {}
@@ -102,6 +113,6 @@ def load_tensors(
     for path, names in by_file.items():
         with safe_open(path, framework="pt", device="cpu") as fh:
             for name in names:
-                dtype = target_dtype(stored[name], specs[name].kind, act_dtype, name)
+                dtype = target_dtype(stored[name], specs[name].kind, act_dtype, name, specs[name].precision, keep_float32)
                 out[name] = fh.get_tensor(name).to(device=device, dtype=dtype).contiguous()
     return out

@@ -16,8 +16,8 @@ import torch
 from helpers import cache_layout
 
 
-def embedding(tokens, table):
-    return table[tokens.long()].float()
+def embedding(tokens, table, scale=1.0):
+    return table[tokens.long()].float() * scale
 
 
 def add_rmsnorm(h, delta, weight, eps, out_dtype, rows=None):

@@ -168,19 +168,36 @@ def test_random_folder_round_trip(tmp_path):
     assert 0.5 <= float(stored["norm.weight"].float().min()) and float(stored["norm.weight"].float().max()) <= 1.5
 
 
-def test_tensors_stored_in_32_bits_stay_so(tmp_path):
+def test_types_after_loading_in_bfloat16_mode(tmp_path):
+    """Matrices stored in 32 bits are cast to bfloat16, as the reference casts every parameter
+    (cwm/model/parallelize_transformer.py:50-59), so that every product runs on the bfloat16
+    kernels; a tensor whose spec keeps its stored precision (norm weights) stays float32; with
+    keep_float32 every tensor stored in 32 bits stays so; float16 becomes bfloat16."""
     from safetensors.torch import save_file
+    from cwm_amd.engine import load_model
     from cwm_amd.weights import load_tensors
 
-    folder = models.make_folder(tmp_path, "tiny_a", seed=1, dtype="bfloat16")
+    folder = models.make_folder(tmp_path, "tiny_a", seed=1, dtype="float32")
     _, stored = models.read_folder(folder)
-    stored["norm.weight"] = stored["norm.weight"].float()
-    stored["layers.0.attention.wq.weight"] = stored["layers.0.attention.wq.weight"].to(torch.float16)
+    assert all(t.dtype == torch.float32 for t in stored.values())
+    stored["layers.0.attention.wk.weight"] = stored["layers.0.attention.wk.weight"].to(torch.float16)
     save_file(stored, os.path.join(folder, "model.safetensors"))
-    got = load_tensors(folder, _specs("tiny_a"), torch.bfloat16, torch.device("cpu"))
-    assert got["norm.weight"].dtype == torch.float32
-    assert got["layers.0.attention.wq.weight"].dtype == torch.bfloat16
-    assert got["output.weight"].dtype == torch.bfloat16
+    specs = _specs("tiny_a")
+    got = load_tensors(folder, specs, torch.bfloat16, torch.device("cpu"))
+    for name, t in got.items():
+        want = torch.float32 if specs[name].precision == "stored" else torch.bfloat16
+        assert t.dtype == want, name
+    assert got["norm.weight"].dtype == torch.float32 and got["layers.1.ffn_norm.weight"].dtype == torch.float32
+    assert got["layers.0.attention.wq.weight"].dtype == torch.bfloat16 and got["tok_embeddings.weight"].dtype == torch.bfloat16
+    assert torch.equal(got["output.weight"], stored["output.weight"].bfloat16())
+    kept = load_tensors(folder, specs, torch.bfloat16, torch.device("cpu"), keep_float32=True)
+    assert kept["layers.0.attention.wq.weight"].dtype == torch.float32
+    assert kept["layers.0.attention.wk.weight"].dtype == torch.bfloat16  # stored in 16 bits
+    # through the model: the joined projections are bfloat16
+    model, _ = load_model(folder, "bfloat16", "cpu")
+    assert model.blocks[0].mixer.qkv.weight.dtype == torch.bfloat16
+    assert model.blocks[0].feed_forward.gate_up.weight.dtype == torch.bfloat16
+    assert model.blocks[0].norm1.weight.dtype == torch.float32
 
 
 def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):

@@ -320,3 +320,170 @@ def test_toy_position_encoding_registers_and_reaches_the_kernels(dtype):
         assert (other - want).abs().max() > 10 * tol * want.abs().max()
     finally:
         del POSITION_ENCODINGS["toy_half_linear"]
+
+
+# ---- rotation of the halves of a head, and a norm between projection and rotation -------------------- #
+def _rotate_halves(x, positions, freqs):
+    """Element i of a head turns with element i + head_dim / 2 by positions * freqs[i]."""
+    half = x.shape[-1] // 2
+    ang = positions.double()[:, None] * freqs.double()[None, :]
+    cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    a, b = x[..., :half], x[..., half:]
+    return torch.cat([a * cos - b * sin, b * cos + a * sin], dim=-1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_toy_halves_rotation_and_a_norm_before_it(dtype):
+    """Two things that the framework's own architecture does not have, added from here: a rotary
+    encoding that pairs element i with i + head_dim / 2 (it only says so; the attention part
+    reorders its projections' rows once and the kernels stay as they are), and an attention
+    that normalises every query and key head between projection and rotation (the seam
+    `transform_qk`; such steps run the projection, the hook and the rotation + cache write one
+    after the other).  Prefill and decode against the plain attention on whole sequences."""
+    from cwm_amd.cache import CacheManager, CacheStorage
+    from cwm_amd.engine import Portion
+    from cwm_amd.engine.batch import build_batch
+    from cwm_amd.parts import PartChoice, PositionEncoding, Runtime, register_part
+    from cwm_amd.parts.attention import PagedAttention
+    from cwm_amd.parts.base import MIXERS, POSITION_ENCODINGS
+    from cwm_amd.weights import random_tensors
+
+    theta = 200.0
+
+    class HalvesRotary(PositionEncoding):
+        def __init__(self, head_dim):
+            self.head_dim = head_dim
+
+        def bind(self, tensors, runtime):
+            super().bind(tensors, runtime)
+            self.table = plain.rope_frequencies(self.head_dim, theta).to(runtime.device)
+
+        def rotary_table(self):
+            return self.table
+
+        def rotary_pairing(self):
+            return "halves"
+
+    class UnitNormAttention(PagedAttention):
+        def transform_qk(self, q, k, batch):
+            for t in (q, k):
+                if t is not None:
+                    t.copy_(torch.nn.functional.normalize(t.float(), dim=-1).to(t.dtype))
+
+    register_part("position_encoding", "toy_halves", HalvesRotary)
+    register_part("mixer", "toy_unit_norm_attention", UnitNormAttention)
+    try:
+        dim, n_heads, n_kv, hd = 40, 6, 2, 16
+        for mixer_name, normalise in (("paged_attention", False), ("toy_unit_norm_attention", True)):
+            scale = 4.0 if normalise else 0.3
+            choice = PartChoice(mixer_name, {"dim": dim, "n_heads": n_heads, "n_kv_heads": n_kv, "head_dim": hd, "scale": scale, "bias": True,
+                                             "position_encoding": PartChoice("toy_halves", {"head_dim": hd})})
+            part = choice.build("mixer")
+            runtime = Runtime(torch.device("cuda:0"), dtype)
+            host = random_tensors(part.tensor_specs(), seed=13, std=0.4, norm_init="ones", dtype=dtype)
+            part.bind({k: v.to("cuda:0") for k, v in host.items()}, runtime)
+
+            n = 23
+            x = (torch.randn(n, dim, generator=torch.Generator().manual_seed(4)) * 0.5).to(dtype)
+            w = {k: v.double() for k, v in host.items()}
+            xd = x.double()
+            pos = torch.arange(n)
+            freqs = plain.rope_frequencies(hd, theta)
+            q = plain.linear(xd, w["wq.weight"], w["wq.bias"]).view(n, n_heads, hd)
+            k = plain.linear(xd, w["wk.weight"], w["wk.bias"]).view(n, n_kv, hd)
+            v = plain.linear(xd, w["wv.weight"], w["wv.bias"]).view(n, n_kv, hd)
+            if normalise:
+                q, k = torch.nn.functional.normalize(q, dim=-1), torch.nn.functional.normalize(k, dim=-1)
+                if dtype == torch.bfloat16:  # the hook stores what it made
+                    q, k = q.to(dtype).double(), k.to(dtype).double()
+            q, k = _rotate_halves(q, pos, freqs), _rotate_halves(k, pos, freqs)
+            want = plain.linear(plain.attention(q, k, v, window_left=-1, scale=scale).reshape(n, -1), w["wo.weight"]).float()
+            # the pairing matters: adjacent pairs give something else
+            wrong = plain.linear(
+                plain.attention(plain.rope_apply(q, pos, freqs), plain.rope_apply(k, pos, freqs), v, window_left=-1, scale=scale).reshape(n, -1),
+                w["wo.weight"],
+            ).float()
+
+            manager = CacheManager([part.cache_spec()], 8, 8, 2)
+            storage = CacheStorage(manager, runtime.device, dtype)
+            manager.admit("r")
+            got = []
+            for start, count in ((0, 14), (14, 1), (15, 1), (16, 7)):
+                assert manager.extend("r", count)
+                batch = build_batch([Portion("r", [0] * count, [])], manager, runtime.device, vocab_size=10)
+                out = part.forward(x[start : start + count].to("cuda:0"), batch, storage.view(0, batch))
+                if out.dim() == 3:
+                    out = out.sum(0)
+                got.append(out.float().cpu())
+                manager.advance("r", count)
+            got = torch.cat(got)
+            tol = 2e-5 if dtype == torch.float32 else 3e-2
+            assert (got - want).abs().max() <= tol * want.abs().max(), mixer_name
+            assert (wrong - want).abs().max() > 10 * tol * want.abs().max()
+    finally:
+        del POSITION_ENCODINGS["toy_halves"]
+        del MIXERS["toy_unit_norm_attention"]
+
+
+def test_toy_model_with_tied_head_scaled_embedding_and_two_kinds_of_norm():
+    """A plan may tie the output projection to the embedding table, scale the embedding, and give a
+    layer's two norms different constants; none of it is in the framework's own architecture.  One
+    layer, float32, against the same computation from the plain parts."""
+    from cwm_amd.config import ARCHITECTURES, parse_config, register_architecture
+    from cwm_amd.models import Model
+    from cwm_amd.parts import LayerCall, LayerPlan, ModelPlan, PartChoice, Runtime
+    from cwm_amd.weights import random_tensors
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        architecture: str
+        dim: int
+        vocab_size: int
+
+    n_heads, n_kv, hd, theta, eps1, eps2, emb_scale = 2, 1, 16, 80.0, 1e-5, 0.5, 3.0
+
+    def toy_plan(cfg):
+        rope = PartChoice("rotary", {"head_dim": hd, "theta": theta})
+        attn = PartChoice("paged_attention", {"dim": cfg.dim, "n_heads": n_heads, "n_kv_heads": n_kv, "head_dim": hd, "scale": hd**-0.5,
+                                              "position_encoding": rope})
+        names = {"norm1": "n1.", "mixer": "attn.", "norm2": "n2.", "feed_forward": "ff."}
+        layer = LayerPlan("l0.", "pre_norm", PartChoice("rmsnorm", {"dim": cfg.dim, "eps": eps1}), attn,
+                          PartChoice("swiglu", {"dim": cfg.dim, "hidden_dim": 40}), names,
+                          norm2=PartChoice("rmsnorm", {"dim": cfg.dim, "eps": eps2}))
+        return ModelPlan(cfg.vocab_size, cfg.dim, "emb", [layer], [LayerCall(0)], PartChoice("rmsnorm", {"dim": cfg.dim, "eps": eps1}),
+                         "final", "unused", embedding_scale=emb_scale, tied_head=True)
+
+    register_architecture("toy_tied_model", ToyConfig, toy_plan)
+    try:
+        arch, cfg = parse_config({"architecture": "toy_tied_model", "dim": 32, "vocab_size": 59})
+        model = Model(arch.build_plan(cfg))
+        assert "unused.weight" not in model.tensor_specs() and "emb.weight" in model.tensor_specs()
+        runtime = Runtime(torch.device("cuda:0"), torch.float32)
+        host = random_tensors(model.tensor_specs(), seed=6, std=0.3, norm_init="uniform", dtype=torch.float32)
+        model.bind({k: v.to("cuda:0") for k, v in host.items()}, runtime)
+
+        def whole_sequence(tokens):
+            w = {k: v.double() for k, v in host.items()}
+            n = len(tokens)
+            pos = torch.arange(n)
+            freqs = plain.rope_frequencies(hd, theta)
+            h = emb_scale * w["emb.weight"][torch.tensor(tokens)]
+            x = plain.rms_norm(h, w["l0.n1.weight"], eps1)
+            q = plain.rope_apply(plain.linear(x, w["l0.attn.wq.weight"]).view(n, n_heads, hd), pos, freqs)
+            k = plain.rope_apply(plain.linear(x, w["l0.attn.wk.weight"]).view(n, n_kv, hd), pos, freqs)
+            v = plain.linear(x, w["l0.attn.wv.weight"]).view(n, n_kv, hd)
+            h = h + plain.linear(plain.attention(q, k, v, scale=hd**-0.5).reshape(n, -1), w["l0.attn.wo.weight"])
+            x = plain.rms_norm(h, w["l0.n2.weight"], eps2)
+            h = h + plain.swiglu(x, w["l0.ff.w1.weight"], w["l0.ff.w2.weight"], w["l0.ff.w3.weight"])
+            return plain.linear(plain.rms_norm(h, w["final.weight"], eps1), w["emb.weight"]).float()
+
+        toks = {"a": traces.random_tokens(3, 19, 59), "b": traces.random_tokens(4, 11, 59)}
+        cut = _step_through(model, runtime, toks, [{"a": 4, "b": 1}, {"a": 1, "b": 6}, {"a": 14, "b": 4}])
+        for k in toks:
+            torch.testing.assert_close(cut[k], whole_sequence(toks[k]), rtol=2e-4, atol=2e-4)
+        # eps2 = 0.5 is no small number: with eps1 in its place the logits differ
+        eps2_saved, eps2 = eps2, eps1
+        assert not torch.allclose(cut["a"], whole_sequence(toks["a"]), rtol=1e-2, atol=1e-2)
+        eps2 = eps2_saved
+    finally:
+        del ARCHITECTURES["toy_tied_model"]
