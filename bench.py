@@ -8,9 +8,16 @@ requests at a context of 32,768 tokens each; a step is one decode step of the wh
 batch through the engine's step function and sampler.  It prints one JSON line:
 `value` is decoded tokens a second; `prefill` is a 2,048-token prompt in one step;
 `roofline` compares the bytes a decode step has to read (every weight once, and the
-cache of the live requests) with the HBM peak; `points` holds decoding at batch 1
-and 64 with 1,024-token contexts.  The cache of the timed requests is filled with
-random numbers instead of being computed (the weights are random too).
+cache of the live requests) with the HBM peak.  The cache of the timed requests is filled
+with random numbers instead of being computed (the weights are random too).
+
+`points` holds the workload that the baseline names: batches of 1, 8 and 64 requests with
+prompts of 1,024 random tokens and 256 new tokens each, through `Engine.step` (scheduler,
+step function and sampler, a host round trip per step); `decode_b<N>` is N times the number
+of steps in which all N requests decode, over the time of those steps; `decode_b<N>_ms` is the
+median of their times and `decode_b<N>_frac` the bytes such a step has to read over that
+median and the HBM peak.  `decode_b8_ctx<C>` are decode steps of 8 requests at other context
+lengths through the step function, as the headline.
 """
 
 from __future__ import annotations
@@ -121,29 +128,43 @@ def main() -> int:
     if args.serve:
         return serve_run(args, model, typed, shape_name)
     esize = 2 if args.dtype == "bf16" else 4
+    # what a step reads of the weights, from the model's own list of tensors: everything but the embedding
+    # table (of which a step reads one row a token); `matrix_params` are the entries of the matrices, which
+    # every token is multiplied with
     weight_bytes = 0
-    for blk in model.blocks:
-        for lin in (blk.mixer.qkv, blk.mixer.wo, blk.feed_forward.gate_up, blk.feed_forward.down):
-            weight_bytes += lin.weight.numel() * lin.weight.element_size()
-        weight_bytes += 2 * model.dim * blk.norm1.weight.element_size()
-    weight_bytes += model.head.weight.numel() * model.head.weight.element_size()
-    window = typed.window_attn.local_window if typed.window_attn is not None else None
+    matrix_params = 0
+    head_params = 0
+    embedding = model.plan.embedding_name + ".weight"
+    for name, spec in model.tensor_specs().items():
+        count = 1
+        for n in spec.shape:
+            count *= n
+        if name == embedding and not model.plan.tied_head:
+            continue
+        weight_bytes += count * esize
+        if len(spec.shape) == 2:
+            if name == embedding or name == model.plan.head_name + ".weight":
+                head_params += count
+            else:
+                matrix_params += count
+    windows = sorted({spec.window for spec in model.cache_specs if isinstance(spec, PagedKVSpec) and spec.window is not None})
+    window = windows[0] if windows else None
     page = args.page
     sampler = Sampler(device)
     vocab = typed.vocab_size
 
     def cache_bytes(batch, ctx):
-        per_layer_token = 2 * typed.kv_heads * typed.head_size * esize
         total = 0
         for spec in model.cache_specs:
-            keys = ctx if spec.window is None else min(ctx, spec.window)
-            total += batch * keys * per_layer_token
+            if isinstance(spec, PagedKVSpec):
+                keys = ctx if spec.window is None else min(ctx, spec.window)
+                total += batch * keys * 2 * spec.n_kv_heads * spec.head_dim * esize
         return total
 
     def make_runner(batch, ctx, extra):
         pages = {None: batch * ((ctx + extra + page - 1) // page + 1)}
-        if window is not None:
-            pages[window] = batch * ((min(ctx, window) + extra + 2 * page - 1) // page + 2)
+        for w in windows:
+            pages[w] = batch * ((min(ctx, w) + extra + 2 * page - 1) // page + 2)
         manager = CacheManager(model.cache_specs, page, pages, batch)
         storage = CacheStorage(manager, device, model.runtime.act_dtype)
         for t in storage.paged.values():
@@ -211,15 +232,15 @@ def main() -> int:
 
     n_prefill = 2048
     prefill_s = prefill_run(n_prefill)
-    linear_params = sum(
-        lin.weight.numel() for blk in model.blocks for lin in (blk.mixer.qkv, blk.mixer.wo, blk.feed_forward.gate_up, blk.feed_forward.down)
-    )
     attn_flops = 0
-    for spec in model.cache_specs:
-        # causal: token p reads min(p + 1, window) keys; 2 products (QK^T and PV) of 2 flops
-        keys = sum(min(p + 1, spec.window or (p + 1)) for p in range(n_prefill))
-        attn_flops += 4 * keys * typed.n_heads * typed.head_size
-    prefill_flops = 2 * n_prefill * linear_params + attn_flops + 2 * model.head.weight.numel()
+    for call, slot in zip(model.run_order, model.cache_slot):
+        spec = model.cache_specs[slot]
+        if isinstance(spec, PagedKVSpec):
+            # causal: token p reads min(p + 1, window) keys; 2 products (QK^T and PV) of 2 flops, for every query head
+            keys = sum(min(p + 1, spec.window or (p + 1)) for p in range(n_prefill))
+            query_heads = getattr(model.blocks[call.layer].mixer, "n_heads", spec.n_kv_heads)
+            attn_flops += 4 * keys * query_heads * spec.head_dim
+    prefill_flops = 2 * n_prefill * matrix_params + attn_flops + 2 * head_params
     prefill = {
         "value": round(n_prefill / prefill_s, 1),
         "tokens": n_prefill,
@@ -229,8 +250,16 @@ def main() -> int:
 
     points = {}
     if not args.no_points:
-        for b in (1, 64):
-            points[f"decode_b{b}"] = round(decode_run(b, 1024, max(5, args.steps // 2), 2)[0], 1)
+        for ctx in (8192, 131072):
+            if ctx != args.context:
+                points[f"decode_b{args.batch}_ctx{ctx}"] = round(decode_run(args.batch, ctx, 10, 2)[0], 1)
+        for b in (1, 8, 64):
+            tok_s_b, median_ms, n_steps = engine_point(model, b, 1024, 256, page, typed.vocab_size)
+            bytes_b = weight_bytes + cache_bytes(b, 1024 + 128)  # the context grows from 1,024 to 1,280 over the run
+            points[f"decode_b{b}"] = round(tok_s_b, 1)
+            points[f"decode_b{b}_ms"] = round(median_ms, 3)
+            points[f"decode_b{b}_frac"] = round(bytes_b / (median_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+            points[f"decode_b{b}_steps"] = n_steps
 
     line = {
         "metric": f"decode tok/s ({shape_name.split(' (')[0]}, batch {args.batch}, context {args.context})",
@@ -260,7 +289,8 @@ def main() -> int:
             "vocab_size": typed.vocab_size,
             "local_window": window or 0,
             "page_size": page,
-            "points_context": 1024,
+            "points_prompt_tokens": 1024,
+            "points_new_tokens": 256,
             "prefill_tokens": n_prefill,
         },
         "prefill": prefill,
@@ -275,6 +305,42 @@ def main() -> int:
     }
     print(json.dumps(line), flush=True)
     return 0
+
+
+def engine_point(model, batch, prompt_tokens, new_tokens, page, vocab):
+    """`batch` requests with prompts of `prompt_tokens` random tokens and `new_tokens` new tokens each
+    through the engine (scheduler, step function, sampler).  Returns (decoded tokens a second over the
+    steps in which all `batch` requests decode, the median time of such a step in ms, their number)."""
+    import random
+    import statistics
+
+    import torch
+
+    from cwm_amd.engine import Engine, GenArgs, Packet
+
+    rng = random.Random(batch)
+    gen_args = GenArgs(
+        use_sampling=True, temperature=0.7, top_p=1.0, max_batch=batch, cache_block=page, max_prefill=4096,
+        max_seq=batch * (prompt_tokens + new_tokens + 2 * page),
+    )
+    engine = Engine(gen_args, model)
+    for i in range(batch):
+        engine.submit(Packet(thread_id=i, tokens=[rng.randrange(vocab) for _ in range(prompt_tokens)], max_gen=new_tokens))
+    times = []
+    finished = 0
+    torch.cuda.synchronize()
+    while engine.scheduler.has_work():
+        start = time.perf_counter()
+        finished += len(engine.step())
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - start
+        if engine.last_step_sequences == batch and engine.last_step_tokens == batch:
+            times.append(elapsed)
+    assert finished == batch
+    del engine
+    torch.cuda.empty_cache()
+    times = times[2:] if len(times) > 8 else times  # the first such steps still build their plans and buffers
+    return batch * len(times) / sum(times), 1e3 * statistics.median(times), len(times)
 
 
 def serve_run(args, model, typed, shape_name) -> int:
@@ -294,7 +360,8 @@ def serve_run(args, model, typed, shape_name) -> int:
         temperature=0.7,
         top_p=0.95,
         max_batch=min(args.serve, 64),
-        max_seq=sum(lengths) + args.serve * (args.new + 2 * args.page),
+        max_seq=-1,  # the pools take what is free on the device
+        expected_seq=4096 + args.new,
         cache_block=args.page,
         max_prefill=4096,
     )

@@ -154,6 +154,8 @@ class Engine:
         self.n_sequences = 0
         self.n_generated = 0
         self._reported = 0
+        self.last_step_tokens = 0  # tokens and sequences that the latest step ran
+        self.last_step_sequences = 0
 
     # ---- construction ------------------------------------------------------------ #
     @classmethod
@@ -289,6 +291,8 @@ class Engine:
         for item in batch:
             if item.start == 0 and item.request.cached == 0:
                 self.storage.zero_state(self.manager.slot(item.request.rid))
+        self.last_step_sequences = len(batch)
+        self.last_step_tokens = sum(item.count for item in batch)
         if batch:
             logits = self.runner.step(sched.portions(batch))
             self.n_steps += 1
