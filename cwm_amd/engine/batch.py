@@ -121,21 +121,27 @@ def build_batch(
     page_size = manager.page_size
     width = max(1, max((kv + page_size - 1) // page_size for kv in kv_lens))
     tables = []
+    columns = np.arange(width, dtype=np.int64)[None, :]
+    last_page = np.asarray([pages_for(kv, page_size) for kv in kv_lens], dtype=np.int64)[:, None]
     for g in manager.groups:
         tbl = np.full((n_seqs, width), -1, dtype=np.int32)
         for b, rid in enumerate(rids):
             pages = manager.table(g.index, rid)
             n = min(len(pages), width)
             tbl[b, :n] = pages[:n]
-            # every page that this step's queries can read, or that its tokens are written to, is held
-            first = first_page_needed(kv_lens[b] - q_lens[b], g.window, page_size)
-            last = pages_for(kv_lens[b], page_size)
-            span = tbl[b, first:last]
-            if span.size != last - first or (span < 0).any() or (span >= g.pool.num_pages).any():
-                raise BatchError(
-                    f"request {rid!r}: group {g.index} holds no page for some of the logical pages {first}..{last - 1} "
-                    f"that this step reads or writes (table {span.tolist()}, pool of {g.pool.num_pages})"
-                )
+        # every page that this step's queries can read, or that its tokens are written to, is held
+        first_page = np.asarray(
+            [first_page_needed(kv - q, g.window, page_size) for kv, q in zip(kv_lens, q_lens)], dtype=np.int64
+        )[:, None]
+        needed = (columns >= first_page) & (columns < last_page)
+        bad = needed & ((tbl < 0) | (tbl >= g.pool.num_pages))
+        if bad.any():
+            b = int(np.argmax(bad.any(axis=1)))
+            first, last = int(first_page[b, 0]), int(last_page[b, 0])
+            raise BatchError(
+                f"request {rids[b]!r}: group {g.index} holds no page for some of the logical pages {first}..{last - 1} "
+                f"that this step reads or writes (table {tbl[b, first:last].tolist()}, pool of {g.pool.num_pages})"
+            )
         tables.append(tbl)
 
     # one buffer, one copy

@@ -67,6 +67,15 @@ class Request:
     def __len__(self) -> int:
         return len(self.prompt) + len(self.generated)
 
+    def tokens_between(self, start: int, end: int) -> List[int]:
+        """all_tokens()[start:end] without joining the two lists (a decoded token is one element)."""
+        n = len(self.prompt)
+        if end <= n:
+            return self.prompt[start:end]
+        if start >= n:
+            return self.generated[start - n : end - n]
+        return self.prompt[start:] + self.generated[: end - n]
+
     @property
     def pending(self) -> int:
         """Known tokens not yet in the cache."""
@@ -244,7 +253,7 @@ class Scheduler:
         out = []
         for item in batch:
             request = item.request
-            toks = request.all_tokens()[item.start : item.start + item.count]
+            toks = request.tokens_between(item.start, item.start + item.count)
             item.prompt_places = []
             if request.want_prompt_logprobs:
                 # prompt positions not scored yet (a recomputed request has its scores already)

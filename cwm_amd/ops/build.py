@@ -1,7 +1,7 @@
 """Compiles the HIP sources under `cwm_amd/csrc` for gfx950 and loads them.
 
 Each source file becomes one shared library next to the package
-(`cwm_amd/_lib/<name>[__DEF=VAL...].so`), built with plain `hipcc` and loaded with
+(`cwm_amd/_lib/<name>[__DEF_VAL...].so`), built with plain `hipcc` and loaded with
 ctypes.  A library is built when it is first asked for and is missing or older than
 its sources (a digest of the sources and flags is kept beside it), so a fresh
 checkout compiles exactly the kernels that the model at hand uses.  While hipcc
@@ -105,7 +105,7 @@ def _choose_lib_dir() -> str:
 
 
 def _variant_tag(defines: Mapping[str, int]) -> str:
-    return "".join(f"__{k}={defines[k]}" for k in sorted(defines))
+    return "".join(f"__{k}_{defines[k]}" for k in sorted(defines))  # letters, digits and underscores only: a plain file name
 
 
 def _digest(name: str, defines: Mapping[str, int]) -> str:

@@ -70,3 +70,62 @@ def test_a_step_whose_readable_pages_are_not_all_held_is_refused():
         build_batch([Portion("a", [1, 2, 3], [2])], manager, device, 50)
     manager.table(0, "a")[0] = held
     build_batch([Portion("a", [1, 2, 3], [2])], manager, device, 50)
+
+
+def test_trace_run_options(tmp_path, monkeypatch, capsys):
+    """The replay program with a configuration and a seed instead of a folder, pages of 8 tokens,
+    the pools' sizes given outright, and the log of pages taken and given back: a window group
+    gives pages back while its request runs, and no page is handed out while it is held."""
+    import io
+    import json
+    import sys
+
+    from cwm_amd import replay
+
+    cpu_ops.install(monkeypatch)
+    config = configs.get("tiny_b")
+    cfg_path = tmp_path / "config.json"
+    cfg_path.write_text(json.dumps(config))
+    vocab = config["vocab_size"]
+    requests = _requests(vocab, [40, 23], seed=5)
+    steps = traces.portions(requests, sizes=[5, 3, 9])
+    log = tmp_path / "pages.jsonl"
+    out = tmp_path / "out"
+    monkeypatch.setattr(sys, "stdin", io.StringIO("".join(json.dumps(s) + "\n" for s in steps)))
+    rc = replay.main([
+        "--random-config", str(cfg_path), "--seed", "3", "--std", "0.05", "--dtype", "float32", "--out", str(out), "--max-tokens", "64",
+        "--device", "cpu", "--page-size", "8", "--pages", "all=6,8=3", "--page-log", str(log),
+    ])
+    assert rc == 0
+    assert [l for l in capsys.readouterr().out.splitlines() if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+    # the logits are those of the plain implementation on the same random weights
+    from cwm_amd.weights import write_random_model
+
+    folder = str(tmp_path / "same")
+    write_random_model(folder, config, seed=3, std=0.05, norm_init="ones", dtype="float32")
+    outputs = {s["step"]: np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(-1, vocab) for s in steps}
+    got = traces.gather(steps, outputs, {k: len(v) for k, v in requests.items()}, vocab)
+    want = models.plain_logits(folder, requests, dtype=torch.float32)
+    for rid in requests:
+        np.testing.assert_allclose(got[rid], want[rid], rtol=2e-4, atol=2e-5)
+    # the log: what is taken was free, what is given back was held
+    records = [json.loads(l) for l in log.read_text().splitlines()]
+    assert len(records) == len(steps)
+    held = {0: set(), 1: set()}
+    sizes = {0: None, 1: None}
+    gave_back_early = False
+    for rec, st in zip(records, steps):
+        for rid, by_group in rec["take"].items():
+            for g, pages in by_group.items():
+                assert not held[int(g)] & set(pages)
+                held[int(g)] |= set(pages)
+        for g, pages in rec["give"].items():
+            assert set(pages) <= held[int(g)]
+            held[int(g)] -= set(pages)
+            if not st["end"]:
+                gave_back_early = True
+        assert len(rec["free"]) == 2
+    assert gave_back_early  # the window of 8 keys passes pages of 8 tokens as the request goes on
+    assert held == {0: set(), 1: set()}
+    with pytest.raises(SystemExit):
+        replay.main(["--dtype", "float32", "--out", str(out), "--max-tokens", "64"])
