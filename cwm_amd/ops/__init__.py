@@ -228,6 +228,71 @@ def gemm_f32(
     return out
 
 
+F32_STREAM_MAX_ROWS = 16
+_f32_stream_block_steps: Optional[int] = None
+
+
+def _f32_stream_takes(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    return (
+        x.dtype == torch.float32 and weight.dtype == torch.float32
+        and x.dim() == 2 and weight.dim() == 2 and x.shape[0] <= F32_STREAM_MAX_ROWS
+        and x.shape[1] % 4 == 0 and x.stride(-1) == 1 and weight.stride(-1) == 1
+        and (x.shape[0] <= 1 or x.stride(0) % 4 == 0) and (weight.shape[0] <= 1 or weight.stride(0) % 4 == 0)
+        and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
+    )
+
+
+def gemm_f32_stream(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    out_dtype: Optional[torch.dtype] = None,
+    partials_ok: bool = False,
+) -> torch.Tensor:
+    """float32 x [M <= 16, K] @ float32 weight[N, K]^T with float32 multiply-add, the weight
+    streamed once by persistent blocks (the decode-step product of the 32-bit path).  Returns
+    [M, N]; with `partials_ok` it may return float32 partial sums [P, M, N] of a split K."""
+    global _f32_stream_block_steps
+    _need_gpu(x, weight, bias)
+    if not _f32_stream_takes(x, weight) or x.shape[1] != weight.shape[1]:
+        raise KernelError(
+            f"the float32 streaming product takes float32 x [M <= {F32_STREAM_MAX_ROWS}, K] and weight [N, K] with K a multiple "
+            f"of 4 and 16-byte aligned rows; got {tuple(x.shape)} {x.dtype} and {tuple(weight.shape)} {weight.dtype}"
+        )
+    m, k = x.shape
+    n = weight.shape[0]
+    if bias is not None and (bias.shape != (n,) or not bias.is_contiguous()):
+        raise KernelError(f"gemm: bias {tuple(bias.shape)} does not fit {n} outputs")
+    out_dtype = out_dtype or torch.float32
+    lib = _build.load("gemm_f32_stream")
+    if _f32_stream_block_steps is None:
+        _f32_stream_block_steps = int(lib.cwm_gemm_f32_stream_steps_per_block())
+    steps = (k + 15) // 16
+    n_tiles = (n + 15) // 16
+    cus = _compute_units(x.device)
+    k_split = -(-steps // _f32_stream_block_steps)  # K longer than one block's registers is split
+    if partials_ok:
+        while n_tiles * k_split < 2 * cus and k_split < 8 and steps >= 2 * k_split * 16:
+            k_split *= 2  # too few tiles to fill the chip
+    blocks = max(k_split, min(cus, n_tiles * k_split) // k_split * k_split)
+    if k_split == 1:
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    else:
+        out = torch.empty((k_split, m, n), dtype=torch.float32, device=x.device)
+    _check(
+        lib,
+        lib.cwm_gemm_f32_stream(
+            _ptr(x), ctypes.c_long(x.stride(0) if m > 1 else k), _ptr(weight), ctypes.c_long(weight.stride(0) if n > 1 else k),
+            _ptr(out), ctypes.c_int(_code(out.dtype)), ctypes.c_long(n), ctypes.c_long(m * n),
+            _ptr(bias), ctypes.c_int(_code(bias.dtype) if bias is not None else F32),
+            ctypes.c_int(m), ctypes.c_int(n), ctypes.c_int(k), ctypes.c_int(k_split), ctypes.c_int(blocks), _stream(),
+        ),
+    )
+    if k_split > 1 and not partials_ok:
+        return sum_partials(out, out_dtype)
+    return out
+
+
 def linear(
     x: torch.Tensor,
     weight: torch.Tensor,
@@ -237,13 +302,16 @@ def linear(
 ) -> torch.Tensor:
     """y = x W^T (+ b).  cwm/fastgen/forward.py:593-606.
 
-    float32 activations or float32 weights: the float32 kernel (exact products).
+    float32 activations or float32 weights: the float32 kernels (exact products; up to 16
+    rows of float32 on the weight-streaming one, whose sums differ from the other's by rounding).
     bfloat16 activations and weights: matrix cores with float32 accumulation, the
     library product for many rows.  With `partials_ok` the result may be float32
     partial sums [P, M, N] that the caller adds (see `add_rmsnorm`).
     """
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.float32 or weight.dtype == torch.float32:
+        if x.is_cuda and _f32_stream_takes(x, weight):
+            return gemm_f32_stream(x, weight, bias, out_dtype, partials_ok)
         return gemm_f32(x, weight, bias, out_dtype)
     return gemm_bf16(x, weight, bias, out_dtype, partials_ok)
 
@@ -757,6 +825,7 @@ __all__ = [
     "add_rmsnorm",
     "silu_mul",
     "gemm_f32",
+    "gemm_f32_stream",
     "gemm_bf16",
     "gemm_bf16_stream",
     "sum_partials",

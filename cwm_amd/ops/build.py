@@ -50,6 +50,7 @@ SOURCES: Dict[str, Tuple[Mapping[str, int], ...]] = {
     "rope_kv": ({},),
     "attention_simple": ({},),
     "gemm_f32": ({},),
+    "gemm_f32_stream": ({},),
     "sampling": ({},),
     "gemm_bf16_stream": ({},),
     "attention_mfma": tuple({"HEAD_DIM": hd} for hd in (16, 32, 48, 64, 80, 96, 128, 256)),

@@ -189,6 +189,53 @@ def test_gemm_f32_is_true_float32():
     assert (got - float(k)).abs().min() > 1e-6  # not rounded to 1.0 * 1.0
 
 
+@pytest.mark.parametrize("c_dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(1, 263, 120), (8, 6144, 6144), (5, 64, 64), (16, 509, 296), (7, 130, 4), (3, 1000, 21504), (16, 48, 3080), (2, 7, 40)])
+def test_gemm_f32_stream(c_dtype, m, n, k):
+    """The weight-streaming float32 product for up to 16 rows: against float64, with and without
+    partial sums of a split K, and a row's bits do not depend on how many rows the call has."""
+    from cwm_amd import ops
+
+    a = rnd((m, k), torch.float32, 6)
+    w = rnd((n, k), torch.float32, 7)
+    b = rnd((n,), torch.float32, 8)
+    want = a.double() @ w.double().T + b.double()
+    t = dict(rtol=1e-5, atol=2e-7 * k + 1e-6) if c_dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    got = ops.gemm_f32_stream(a.to(DEV), w.to(DEV), b.to(DEV), out_dtype=c_dtype).cpu()
+    assert got.dtype == c_dtype
+    torch.testing.assert_close(got.double(), want, **t)
+    parts = ops.gemm_f32_stream(a.to(DEV), w.to(DEV), b.to(DEV), out_dtype=c_dtype, partials_ok=True).cpu()
+    if parts.dim() == 3:
+        assert parts.dtype == torch.float32
+        parts = parts.sum(0)
+    torch.testing.assert_close(parts.double(), want, **t)
+    fewer = max(1, m // 2)
+    one = ops.gemm_f32_stream(a[m - fewer :].contiguous().to(DEV), w.to(DEV), b.to(DEV), out_dtype=c_dtype).cpu()
+    assert torch.equal(one, got[m - fewer :])
+    # through `linear`: float32 operands of few rows take this kernel
+    via = ops.linear(a.to(DEV), w.to(DEV), b.to(DEV), c_dtype).cpu()
+    assert torch.equal(via, got)
+
+
+def test_gemm_f32_stream_is_true_float32_and_refuses_what_it_does_not_take():
+    from cwm_amd import ops
+
+    k = 4
+    a = torch.full((2, k), 1.0 + 2.0 ** -20, dtype=torch.float32)
+    w = torch.full((3, k), 1.0 - 2.0 ** -21, dtype=torch.float32)
+    got = ops.gemm_f32_stream(a.to(DEV), w.to(DEV)).cpu().double()
+    want = a.double() @ w.double().T
+    assert (got - want).abs().max() < 1e-7
+    assert (got - float(k)).abs().min() > 1e-6  # not rounded to 1.0 * 1.0
+    with pytest.raises(ops.KernelError):
+        ops.gemm_f32_stream(torch.zeros(17, 8, device=DEV), torch.zeros(4, 8, device=DEV))
+    with pytest.raises(ops.KernelError):
+        ops.gemm_f32_stream(torch.zeros(2, 6, device=DEV), torch.zeros(4, 6, device=DEV))
+    # a row length that is no multiple of 4 goes to the other float32 kernel through `linear`
+    x, y = rnd((3, 6), torch.float32, 1), rnd((5, 6), torch.float32, 2)
+    torch.testing.assert_close(ops.linear(x.to(DEV), y.to(DEV)).cpu().double(), x.double() @ y.double().T, rtol=1e-5, atol=1e-5)
+
+
 def test_gemm_rows_do_not_depend_on_batch():
     from cwm_amd import ops
 
