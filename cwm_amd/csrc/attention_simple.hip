@@ -1,24 +1,39 @@
 // Paged causal attention with grouped heads and an optional sliding window: the
-// plain kernel.  One block of four wavefronts per (token, query head), which take the
-// chunks of 64 keys in turn and join their results at the end; keys are read from the
-// paged cache through the sequence's block table; scores, softmax and the output
-// sum are float32 for either storage type.  It takes any head size up to 256, any
-// page size and any head counts, and is the kernel of the float32 path.
+// plain kernel.  Keys are read from the paged cache through the sequence's block
+// table; scores, softmax and the output sum are float32 for either storage type.
+// It takes any head size up to 256, any page size and any head counts, and is the
+// kernel of the float32 path.
 //
 // Formula (cwm/fastgen/forward.py:638-655): query at absolute position p of its
 // sequence reads keys j with max(0, p - window_left) <= j <= p (window_left < 0:
 // from 0); s_j = (q . k_j) * scale; o = sum_j softmax(s)_j v_j; query head h uses
 // key/value head h / (n_q_heads / n_kv_heads).
 //
-// The order of every sum depends only on the token's own position, so the result
-// for a token is the same bits whatever else is in the batch and however the
-// sequence was cut into steps.
+// One block of four wavefronts per (token, key/value head, up to 8 of its query heads,
+// segment of the keys): a key and a value are loaded once and used for all the block's
+// query heads.  A token's keys are cut into segments by a rule of their number alone
+// (one segment up to 2,048 keys, then ceil(n / 2,048) segments, at most 16, of equal
+// length in chunks of 64); the wavefronts of a block take the segment's chunks of 64
+// keys in turn (scores and softmax: a lane per key; values: a lane per dimension) and join
+// their results at the end in the order of the wavefronts; the segments of a token leave partial results (maximum, sum,
+// unnormalised output) that a second kernel joins in the order of the segments.
+//
+// The order of every sum depends only on the token's own position and the window, so
+// the result for a token is the same bits whatever else is in the batch and however
+// the sequence was cut into steps.
 #include "common.h"
 
 CWM_DEFINE_ERROR_API
 
 #define SIMPLE_MAX_HEAD_DIM 256
-#define SIMPLE_WAVES 4  // wavefronts that share one (token, head): they take its chunks of keys in turn
+#define SIMPLE_WAVES 4      // wavefronts of a block: they take the segment's chunks of keys in turn
+#define SIMPLE_HEADS 8      // query heads of one key/value head that a block serves at once
+#define SIMPLE_SEGMENT 2048 // keys up to which a token has one segment
+#define SIMPLE_MAX_SEGMENTS 16
+#define SIMPLE_D_REGS (SIMPLE_MAX_HEAD_DIM / CWM_WAVE)
+
+extern "C" int cwm_attention_simple_max_segments() { return SIMPLE_MAX_SEGMENTS; }
+extern "C" int cwm_attention_simple_segment_keys() { return SIMPLE_SEGMENT; }
 
 // what one lane of a wavefront wrote to LDS, the wavefront's other lanes read after this
 __device__ __forceinline__ void wave_sync() {
@@ -26,29 +41,52 @@ __device__ __forceinline__ void wave_sync() {
   __builtin_amdgcn_wave_barrier();
 }
 
+// segments of a token that reads n_keys keys, and their length (a multiple of 64)
+__device__ __forceinline__ int segments_of(int n_keys, int& seg_len) {
+  int n_seg = 1;
+  if (n_keys > SIMPLE_SEGMENT) n_seg = min(SIMPLE_MAX_SEGMENTS, (n_keys + SIMPLE_SEGMENT - 1) / SIMPLE_SEGMENT);
+  seg_len = ((n_keys + n_seg - 1) / n_seg + CWM_WAVE - 1) / CWM_WAVE * CWM_WAVE;
+  return n_seg;
+}
+
+// partial result of (token, query head, segment): [head_dim] unnormalised output, then maximum and sum
+#define PARTIAL_STRIDE(hd) ((hd) + 2)
+
 template <typename T>
-__global__ void attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out,
-                                        long out_stride, const T* __restrict__ cache,
-                                        const int* __restrict__ block_table, int table_width,
-                                        const int* __restrict__ positions, const int* __restrict__ seq_of_token,
-                                        int n_q_heads, int n_kv_heads, int head_dim, int page_size, int num_pages,
-                                        int window_left, float scale) {
-  __shared__ __attribute__((aligned(16))) float qs[SIMPLE_MAX_HEAD_DIM];
-  __shared__ float ps_all[SIMPLE_WAVES][CWM_WAVE];
+__global__ void __launch_bounds__(SIMPLE_WAVES * CWM_WAVE)
+attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out, long out_stride,
+                        const T* __restrict__ cache, const int* __restrict__ block_table, int table_width,
+                        const int* __restrict__ positions, const int* __restrict__ seq_of_token, float* __restrict__ partial,
+                        int n_q_heads, int n_kv_heads, int head_groups, int head_dim, int page_size, int num_pages,
+                        int window_left, float scale) {
+  __shared__ __attribute__((aligned(16))) float qs[SIMPLE_HEADS][SIMPLE_MAX_HEAD_DIM];
+  // probabilities of a chunk, key jj at [in0 + jj] (in0: the first key's place in its block of 8 values), so that the
+  // eight of a block lie at a multiple of 8
+  __shared__ __attribute__((aligned(16))) float ps_all[SIMPLE_WAVES][SIMPLE_HEADS][CWM_WAVE + 8];
   __shared__ long long voff_all[SIMPLE_WAVES][CWM_WAVE];
-  __shared__ float part_m[SIMPLE_WAVES], part_l[SIMPLE_WAVES];
-  __shared__ float part_o[SIMPLE_WAVES][SIMPLE_MAX_HEAD_DIM];
+  __shared__ float part_m[SIMPLE_WAVES][SIMPLE_HEADS], part_l[SIMPLE_WAVES][SIMPLE_HEADS];
+  __shared__ float part_o[SIMPLE_WAVES][SIMPLE_HEADS][SIMPLE_MAX_HEAD_DIM];
 
   const int lane = threadIdx.x & (CWM_WAVE - 1);
   const int wave = threadIdx.x / CWM_WAVE;
-  float* ps = ps_all[wave];
-  long long* voff = voff_all[wave];
-  const int t = blockIdx.x / n_q_heads;
-  const int h = blockIdx.x - t * n_q_heads;
-  const int g = h / (n_q_heads / n_kv_heads);
+  const int group = n_q_heads / n_kv_heads;
+  int id = blockIdx.x;
+  const int hg = id % head_groups;
+  id /= head_groups;
+  const int g = id % n_kv_heads;
+  const int t = id / n_kv_heads;
+  const int seg = blockIdx.y;
+  const int h0 = g * group + hg * SIMPLE_HEADS;             // the block's first query head
+  const int nh = min(SIMPLE_HEADS, group - hg * SIMPLE_HEADS);  // and how many it serves
   const int p = positions[t];
   const int b = seq_of_token[t];
   const int start = window_left >= 0 ? max(0, p - window_left) : 0;
+  int seg_len;
+  const int n_seg = segments_of(p - start + 1, seg_len);
+  if (seg >= n_seg) return;
+  const int k0 = start + seg * seg_len;
+  const int k1 = min(p + 1, k0 + seg_len);  // exclusive
+
   const size_t plane = (size_t)n_kv_heads * page_size * head_dim;
   const int v_block = (page_size % 8 == 0) ? 8 : page_size;
   const float neg_inf = -__builtin_inff();
@@ -56,156 +94,314 @@ __global__ void attention_simple_kernel(const T* __restrict__ q, long q_stride, 
   // float32 rows of keys and blocks of values can be read 16 bytes at a time
   const bool vec4 = head_dim % 4 == 0 && ((uintptr_t)cache % 16) == 0;
 
-  const T* qrow = q + (size_t)t * q_stride + (size_t)h * head_dim;
-  for (int d = threadIdx.x; d < head_dim; d += SIMPLE_WAVES * CWM_WAVE) qs[d] = Elem<T>::load(qrow + d);
+  for (int e = threadIdx.x; e < nh * head_dim; e += SIMPLE_WAVES * CWM_WAVE) {
+    const int h = e / head_dim, d = e - h * head_dim;
+    qs[h][d] = Elem<T>::load(q + (size_t)t * q_stride + (size_t)(h0 + h) * head_dim + d);
+  }
   __syncthreads();
 
-  float m = neg_inf, l = 0.f;
-  float o[SIMPLE_MAX_HEAD_DIM / CWM_WAVE] = {0.f, 0.f, 0.f, 0.f};
+  float* ps = &ps_all[wave][0][0];
+  long long* voff = voff_all[wave];
+  float m[SIMPLE_HEADS], l[SIMPLE_HEADS];
+  float o[SIMPLE_HEADS][SIMPLE_D_REGS];
+#pragma unroll
+  for (int h = 0; h < SIMPLE_HEADS; ++h) {
+    m[h] = neg_inf;
+    l[h] = 0.f;
+#pragma unroll
+    for (int r = 0; r < SIMPLE_D_REGS; ++r) o[h][r] = 0.f;
+  }
 
-  // wavefront w takes the chunks of 64 keys w, w + SIMPLE_WAVES, ... counted from `start`
-  for (int base = start + wave * CWM_WAVE; base <= p; base += SIMPLE_WAVES * CWM_WAVE) {
+  // wavefront w takes the chunks of 64 keys w, w + SIMPLE_WAVES, ... of the segment
+  for (int base = k0 + wave * CWM_WAVE; base < k1; base += SIMPLE_WAVES * CWM_WAVE) {
     const int j = base + lane;
-    const bool valid = j <= p;
-    float s = neg_inf;
+    const bool valid = j < k1;
+    const int n = min(CWM_WAVE, k1 - base);
+    const int in0 = base & 7;  // the first key's place in its block of 8 values
+    float s[SIMPLE_HEADS];
+#pragma unroll
+    for (int h = 0; h < SIMPLE_HEADS; ++h) s[h] = neg_inf;
     long long vo = -1;
     if (valid) {
       const int lp = j / page_size;
       const int slot = j - lp * page_size;
       const int page = lp < table_width ? block_table[(size_t)b * table_width + lp] : -1;
       if (page < 0 || page >= num_pages) {
-        s = nan;  // a key that should be there has no page: make it show
+#pragma unroll
+        for (int h = 0; h < SIMPLE_HEADS; ++h) s[h] = nan;  // a key that should be there has no page: make it show
       } else {
         const T* krow = cache + (size_t)page * 2 * plane + ((size_t)g * page_size + slot) * head_dim;
-        float dot = 0.f;
+        float dot[SIMPLE_HEADS];
+#pragma unroll
+        for (int h = 0; h < SIMPLE_HEADS; ++h) dot[h] = 0.f;
         if (sizeof(T) == 4 && vec4) {
-          // four values per load; the sum keeps the order d = 0, 1, 2, ...
-          for (int d = 0; d < head_dim; d += 4) {
+          // sixteen values per round of loads; every sum keeps the order d = 0, 1, 2, ...
+          int d = 0;
+          for (; d + 16 <= head_dim; d += 16) {
+            float4 kv[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) kv[u] = *(const float4*)((const float*)krow + d + 4 * u);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+#pragma unroll
+              for (int h = 0; h < SIMPLE_HEADS; ++h) {
+                if (h < nh) {
+                  const float4 qv = *(const float4*)(&qs[h][d + 4 * u]);
+                  dot[h] = fmaf(qv.x, kv[u].x, dot[h]);
+                  dot[h] = fmaf(qv.y, kv[u].y, dot[h]);
+                  dot[h] = fmaf(qv.z, kv[u].z, dot[h]);
+                  dot[h] = fmaf(qv.w, kv[u].w, dot[h]);
+                }
+              }
+            }
+          }
+          for (; d < head_dim; d += 4) {
             const float4 kv = *(const float4*)((const float*)krow + d);
-            const float4 qv = *(const float4*)(qs + d);
-            dot = fmaf(qv.x, kv.x, dot);
-            dot = fmaf(qv.y, kv.y, dot);
-            dot = fmaf(qv.z, kv.z, dot);
-            dot = fmaf(qv.w, kv.w, dot);
+#pragma unroll
+            for (int h = 0; h < SIMPLE_HEADS; ++h) {
+              if (h < nh) {
+                const float4 qv = *(const float4*)(&qs[h][d]);
+                dot[h] = fmaf(qv.x, kv.x, dot[h]);
+                dot[h] = fmaf(qv.y, kv.y, dot[h]);
+                dot[h] = fmaf(qv.z, kv.z, dot[h]);
+                dot[h] = fmaf(qv.w, kv.w, dot[h]);
+              }
+            }
           }
         } else {
-          for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], Elem<T>::load(krow + d), dot);
+          for (int d = 0; d < head_dim; ++d) {
+            const float kd = Elem<T>::load(krow + d);
+#pragma unroll
+            for (int h = 0; h < SIMPLE_HEADS; ++h)
+              if (h < nh) dot[h] = fmaf(qs[h][d], kd, dot[h]);
+          }
         }
-        s = dot * scale;
+#pragma unroll
+        for (int h = 0; h < SIMPLE_HEADS; ++h) s[h] = dot[h] * scale;
         // values: blocks of v_block keys, [slot / v_block][dim][slot % v_block]
         vo = (long long)((size_t)page * 2 * plane + plane + (size_t)g * head_dim * page_size +
                          (size_t)(slot / v_block) * head_dim * v_block + slot % v_block);
       }
     }
-    const float mx = wave_max(s);
-    const float m_new = fmaxf(m, mx);
-    const float alpha = (m == neg_inf) ? 0.f : expf(m - m_new);
-    const float pj = valid ? expf(s - m_new) : 0.f;
-    l = l * alpha + wave_sum(pj);
-    ps[lane] = pj;
+    float alpha[SIMPLE_HEADS];
+#pragma unroll
+    for (int h = 0; h < SIMPLE_HEADS; ++h) {
+      if (h < nh) {
+        const float mx = wave_max(s[h]);
+        const float m_new = fmaxf(m[h], mx);
+        alpha[h] = (m[h] == neg_inf) ? 0.f : expf(m[h] - m_new);
+        const float pj = valid ? expf(s[h] - m_new) : 0.f;
+        l[h] = l[h] * alpha[h] + wave_sum(pj);
+        ps[h * (CWM_WAVE + 8) + in0 + lane] = pj;
+        m[h] = m_new;
+      } else {
+        alpha[h] = 0.f;
+      }
+    }
     voff[lane] = vo;
     wave_sync();  // the wavefront's own lanes read these next
-    const int n = min(CWM_WAVE, p - base + 1);
 #pragma unroll
-    for (int r = 0; r < SIMPLE_MAX_HEAD_DIM / CWM_WAVE; ++r) {
+    for (int r = 0; r < SIMPLE_D_REGS; ++r) {
       const int d = lane + r * CWM_WAVE;
       if (d < head_dim) {
-        float acc = o[r] * alpha;
-        if (sizeof(T) == 4 && vec4 && v_block == 8) {
-          // the eight keys of a block of values lie side by side for one dimension: two loads serve up
-          // to eight keys; the sum keeps the order of the keys
-          int jj = 0;
-          while (jj < n) {
-            const int in_block = (base + jj) & 7;        // this key's place in its block of 8
-            const int count = min(8 - in_block, n - jj);  // keys of the chunk that lie in this block
-            const long long off = voff[jj];
-            if (off >= 0) {
-              const float* vb = (const float*)cache + (off - in_block) + (size_t)d * 8;
-              const float4 lo = *(const float4*)vb;
-              const float4 hi = *(const float4*)(vb + 4);
-              const float vv[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        float acc[SIMPLE_HEADS];
 #pragma unroll
-              for (int e = 0; e < 8; ++e)
-                if (e >= in_block && e < in_block + count) acc = fmaf(ps[jj + e - in_block], vv[e], acc);
-            } else {
-              for (int e = 0; e < count; ++e) acc = fmaf(ps[jj + e], nan, acc);
+        for (int h = 0; h < SIMPLE_HEADS; ++h) acc[h] = o[h][r] * alpha[h];
+        if (sizeof(T) == 4 && vec4 && v_block == 8) {
+          // the eight keys of a block of values lie side by side for one dimension: two loads serve up to
+          // eight keys.  The chunk's 64 keys lie in at most nine such blocks; all their loads are issued
+          // before the first is used; every sum keeps the order of the keys.
+          float4 lo[9], hi[9];
+#pragma unroll
+          for (int blk = 0; blk < 9; ++blk) {
+            const int jj = max(0, 8 * blk - in0);  // the block's first key of this chunk
+            lo[blk] = hi[blk] = make_float4(nan, nan, nan, nan);
+            if (jj < n && (blk < 8 || in0 > 0)) {
+              const long long off = voff[jj];
+              if (off >= 0) {
+                const float* vb = (const float*)cache + (off - ((base + jj) & 7)) + (size_t)d * 8;
+                lo[blk] = *(const float4*)vb;
+                hi[blk] = *(const float4*)(vb + 4);
+              }
             }
-            jj += count;
+          }
+#pragma unroll
+          for (int blk = 0; blk < 9; ++blk) {
+            if (8 * blk - in0 >= n) break;
+            const float vv[8] = {lo[blk].x, lo[blk].y, lo[blk].z, lo[blk].w, hi[blk].x, hi[blk].y, hi[blk].z, hi[blk].w};
+            float pp[SIMPLE_HEADS][8];
+#pragma unroll
+            for (int h = 0; h < SIMPLE_HEADS; ++h) {
+              if (h < nh) {
+                const float4 pl = *(const float4*)(&ps[h * (CWM_WAVE + 8) + 8 * blk]);
+                const float4 ph = *(const float4*)(&ps[h * (CWM_WAVE + 8) + 8 * blk + 4]);
+                pp[h][0] = pl.x; pp[h][1] = pl.y; pp[h][2] = pl.z; pp[h][3] = pl.w;
+                pp[h][4] = ph.x; pp[h][5] = ph.y; pp[h][6] = ph.z; pp[h][7] = ph.w;
+              }
+            }
+#pragma unroll
+            for (int x = 0; x < 8; ++x) {
+              const int jj = 8 * blk + x - in0;
+              if (jj >= 0 && jj < n) {
+#pragma unroll
+                for (int h = 0; h < SIMPLE_HEADS; ++h)
+                  if (h < nh) acc[h] = fmaf(pp[h][x], vv[x], acc[h]);
+              }
+            }
           }
         } else {
           for (int jj = 0; jj < n; ++jj) {
             const long long off = voff[jj];
             const float vv = off >= 0 ? Elem<T>::load(cache + off + (size_t)d * v_block) : nan;
-            acc = fmaf(ps[jj], vv, acc);
+#pragma unroll
+            for (int h = 0; h < SIMPLE_HEADS; ++h)
+              if (h < nh) acc[h] = fmaf(ps[h * (CWM_WAVE + 8) + in0 + jj], vv, acc[h]);
           }
         }
-        o[r] = acc;
+#pragma unroll
+        for (int h = 0; h < SIMPLE_HEADS; ++h) o[h][r] = acc[h];
       }
     }
     wave_sync();
-    m = m_new;
   }
 
   // the wavefronts' results, joined in the order of the wavefronts
-  if (lane == 0) {
-    part_m[wave] = m;
-    part_l[wave] = l;
-  }
 #pragma unroll
-  for (int r = 0; r < SIMPLE_MAX_HEAD_DIM / CWM_WAVE; ++r) {
-    const int d = lane + r * CWM_WAVE;
-    if (d < head_dim) part_o[wave][d] = o[r];
+  for (int h = 0; h < SIMPLE_HEADS; ++h) {
+    if (h < nh) {
+      if (lane == 0) {
+        part_m[wave][h] = m[h];
+        part_l[wave][h] = l[h];
+      }
+#pragma unroll
+      for (int r = 0; r < SIMPLE_D_REGS; ++r) {
+        const int d = lane + r * CWM_WAVE;
+        if (d < head_dim) part_o[wave][h][d] = o[h][r];
+      }
+    }
   }
   __syncthreads();
-  if (wave != 0) return;
-  float m_all = part_m[0];
+  // wavefront w finishes heads w, w + SIMPLE_WAVES, ...
+  for (int h = wave; h < nh; h += SIMPLE_WAVES) {
+    float m_all = part_m[0][h];
 #pragma unroll
-  for (int w = 1; w < SIMPLE_WAVES; ++w) m_all = fmaxf(m_all, part_m[w]);
-  float weight[SIMPLE_WAVES];
-  float l_all = 0.f;
+    for (int w = 1; w < SIMPLE_WAVES; ++w) m_all = fmaxf(m_all, part_m[w][h]);
+    float weight[SIMPLE_WAVES];
+    float l_all = 0.f;
 #pragma unroll
-  for (int w = 0; w < SIMPLE_WAVES; ++w) {
-    weight[w] = (part_m[w] == neg_inf) ? 0.f : expf(part_m[w] - m_all);  // -inf: that wavefront had no chunk
-    l_all += part_l[w] * weight[w];
-  }
-  T* orow = out + (size_t)t * out_stride + (size_t)h * head_dim;
+    for (int w = 0; w < SIMPLE_WAVES; ++w) {
+      weight[w] = (part_m[w][h] == neg_inf) ? 0.f : expf(part_m[w][h] - m_all);  // -inf: that wavefront had no chunk
+      l_all += part_l[w][h] * weight[w];
+    }
+    T* orow = out + (size_t)t * out_stride + (size_t)(h0 + h) * head_dim;
+    float* prow = n_seg > 1 ? partial + (((size_t)t * n_q_heads + h0 + h) * SIMPLE_MAX_SEGMENTS + seg) * PARTIAL_STRIDE(head_dim) : nullptr;
 #pragma unroll
-  for (int r = 0; r < SIMPLE_MAX_HEAD_DIM / CWM_WAVE; ++r) {
-    const int d = lane + r * CWM_WAVE;
-    if (d < head_dim) {
-      float sum = 0.f;
+    for (int r = 0; r < SIMPLE_D_REGS; ++r) {
+      const int d = lane + r * CWM_WAVE;
+      if (d < head_dim) {
+        float sum = 0.f;
 #pragma unroll
-      for (int w = 0; w < SIMPLE_WAVES; ++w) sum += part_o[w][d] * weight[w];
-      Elem<T>::store(orow + d, sum / l_all);
+        for (int w = 0; w < SIMPLE_WAVES; ++w) sum += part_o[w][h][d] * weight[w];
+        if (n_seg > 1)
+          prow[d] = sum;
+        else
+          Elem<T>::store(orow + d, sum / l_all);
+      }
+    }
+    if (n_seg > 1 && lane == 0) {
+      prow[head_dim] = m_all;
+      prow[head_dim + 1] = l_all;
     }
   }
 }
 
+// Joins the segments of the tokens that have several, in the order of the segments.  One wavefront
+// per (token, query head).
+template <typename T>
+__global__ void __launch_bounds__(CWM_WAVE)
+attention_simple_join_kernel(T* __restrict__ out, long out_stride, const float* __restrict__ partial,
+                             const int* __restrict__ positions, int n_q_heads, int head_dim, int window_left) {
+  const int t = blockIdx.x / n_q_heads;
+  const int h = blockIdx.x - t * n_q_heads;
+  const int lane = threadIdx.x;
+  const int p = positions[t];
+  const int start = window_left >= 0 ? max(0, p - window_left) : 0;
+  int seg_len;
+  const int n_seg = segments_of(p - start + 1, seg_len);
+  if (n_seg <= 1) return;
+  const float neg_inf = -__builtin_inff();
+  const float* base = partial + (((size_t)t * n_q_heads + h) * SIMPLE_MAX_SEGMENTS) * PARTIAL_STRIDE(head_dim);
+  float m_all = neg_inf;
+  for (int s = 0; s < n_seg; ++s) m_all = fmaxf(m_all, base[(size_t)s * PARTIAL_STRIDE(head_dim) + head_dim]);
+  float l_all = 0.f;
+  float o[SIMPLE_D_REGS];
+#pragma unroll
+  for (int r = 0; r < SIMPLE_D_REGS; ++r) o[r] = 0.f;
+  for (int s = 0; s < n_seg; ++s) {
+    const float* prow = base + (size_t)s * PARTIAL_STRIDE(head_dim);
+    const float ms = prow[head_dim];
+    const float weight = (ms == neg_inf) ? 0.f : expf(ms - m_all);
+    l_all += prow[head_dim + 1] * weight;
+#pragma unroll
+    for (int r = 0; r < SIMPLE_D_REGS; ++r) {
+      const int d = lane + r * CWM_WAVE;
+      if (d < head_dim) o[r] += prow[d] * weight;
+    }
+  }
+  T* orow = out + (size_t)t * out_stride + (size_t)h * head_dim;
+#pragma unroll
+  for (int r = 0; r < SIMPLE_D_REGS; ++r) {
+    const int d = lane + r * CWM_WAVE;
+    if (d < head_dim) Elem<T>::store(orow + d, o[r] / l_all);
+  }
+}
+
+// `max_keys`: the most keys that any token of the call reads (its position + 1, or the window if that
+// is less); `partial`: float32 scratch of n_tokens * n_q_heads * 16 * (head_dim + 2) values, needed
+// (and touched) only if max_keys exceeds 2,048.
 extern "C" int cwm_attention_simple(const void* q, long q_stride, void* out, long out_stride, const void* cache,
                                     int dtype, const int* block_table, int table_width, const int* positions,
                                     const int* seq_of_token, int n_tokens, int n_q_heads, int n_kv_heads,
                                     int head_dim, int page_size, int num_pages, int window_left, float scale,
-                                    hipStream_t stream) {
+                                    int max_keys, float* partial, hipStream_t stream) {
   CWM_REQUIRE(n_tokens >= 0, "attention: negative token count");
   CWM_REQUIRE(head_dim > 0 && head_dim <= SIMPLE_MAX_HEAD_DIM, "attention: head_dim %d is outside 1..%d", head_dim,
               SIMPLE_MAX_HEAD_DIM);
   CWM_REQUIRE(n_q_heads > 0 && n_kv_heads > 0 && n_q_heads % n_kv_heads == 0,
               "attention: %d query heads do not divide into %d key/value heads", n_q_heads, n_kv_heads);
   CWM_REQUIRE(page_size > 0 && num_pages > 0 && table_width > 0, "attention: bad cache geometry");
+  CWM_REQUIRE(max_keys >= 1, "attention: max_keys must be at least 1");
   if (n_tokens == 0) return 0;
-  const long long blocks = (long long)n_tokens * n_q_heads;
+  int max_segments = 1;
+  if (max_keys > SIMPLE_SEGMENT) max_segments = (max_keys + SIMPLE_SEGMENT - 1) / SIMPLE_SEGMENT;
+  if (max_segments > SIMPLE_MAX_SEGMENTS) max_segments = SIMPLE_MAX_SEGMENTS;
+  CWM_REQUIRE(max_segments == 1 || partial != nullptr, "attention: more than %d keys need the scratch for partial results",
+              SIMPLE_SEGMENT);
+  const int group = n_q_heads / n_kv_heads;
+  const int head_groups = (group + SIMPLE_HEADS - 1) / SIMPLE_HEADS;
+  const long long blocks = (long long)n_tokens * n_kv_heads * head_groups;
   CWM_REQUIRE(blocks <= 0x7fffffffLL, "attention: too many (token, head) pairs: %lld", blocks);
-  if (dtype == CWM_F32)
-    hipLaunchKernelGGL(attention_simple_kernel<float>, dim3((unsigned)blocks), dim3(SIMPLE_WAVES * CWM_WAVE), 0, stream,
-                       (const float*)q, q_stride, (float*)out, out_stride, (const float*)cache, block_table,
-                       table_width, positions, seq_of_token, n_q_heads, n_kv_heads, head_dim, page_size,
-                       num_pages, window_left, scale);
-  else if (dtype == CWM_BF16)
-    hipLaunchKernelGGL(attention_simple_kernel<bf16_t>, dim3((unsigned)blocks), dim3(SIMPLE_WAVES * CWM_WAVE), 0, stream,
-                       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)cache, block_table,
-                       table_width, positions, seq_of_token, n_q_heads, n_kv_heads, head_dim, page_size,
-                       num_pages, window_left, scale);
-  else
+  const long long join_blocks = (long long)n_tokens * n_q_heads;
+  CWM_REQUIRE(join_blocks <= 0x7fffffffLL, "attention: too many (token, head) pairs: %lld", join_blocks);
+  dim3 grid((unsigned)blocks, (unsigned)max_segments);
+  if (dtype == CWM_F32) {
+    hipLaunchKernelGGL(attention_simple_kernel<float>, grid, dim3(SIMPLE_WAVES * CWM_WAVE), 0, stream, (const float*)q,
+                       q_stride, (float*)out, out_stride, (const float*)cache, block_table, table_width, positions,
+                       seq_of_token, partial, n_q_heads, n_kv_heads, head_groups, head_dim, page_size, num_pages, window_left,
+                       scale);
+    if (max_segments > 1)
+      hipLaunchKernelGGL(attention_simple_join_kernel<float>, dim3((unsigned)join_blocks), dim3(CWM_WAVE), 0, stream,
+                         (float*)out, out_stride, (const float*)partial, positions, n_q_heads, head_dim, window_left);
+  } else if (dtype == CWM_BF16) {
+    hipLaunchKernelGGL(attention_simple_kernel<bf16_t>, grid, dim3(SIMPLE_WAVES * CWM_WAVE), 0, stream, (const bf16_t*)q,
+                       q_stride, (bf16_t*)out, out_stride, (const bf16_t*)cache, block_table, table_width, positions,
+                       seq_of_token, partial, n_q_heads, n_kv_heads, head_groups, head_dim, page_size, num_pages, window_left,
+                       scale);
+    if (max_segments > 1)
+      hipLaunchKernelGGL(attention_simple_join_kernel<bf16_t>, dim3((unsigned)join_blocks), dim3(CWM_WAVE), 0, stream,
+                         (bf16_t*)out, out_stride, (const float*)partial, positions, n_q_heads, head_dim, window_left);
+  } else {
     return cwm_fail("attention: unknown dtype %d", dtype);
+  }
   return cwm_launch_status("attention_simple");
 }

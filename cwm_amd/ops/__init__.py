@@ -584,10 +584,13 @@ def paged_attention_simple(
     seq_of_token: torch.Tensor,
     window: Optional[int],
     scale: float,
+    max_keys: Optional[int] = None,
 ) -> torch.Tensor:
-    """Causal attention of `q` [T, Hq, hd] over the paged cache; one wavefront per
-    (token, head), float32 arithmetic.  `window`: keys read per query, own included
-    (None: all).  Returns [T, Hq * hd]."""
+    """Causal attention of `q` [T, Hq, hd] over the paged cache by the plain kernel:
+    float32 arithmetic, a key/value head's query heads sharing its keys and values, long
+    key ranges cut into segments that a second kernel joins.  `window`: keys read per
+    query, own included (None: all).  `max_keys`: the most keys any token reads (default:
+    from the largest position, which costs a copy to the host).  Returns [T, Hq * hd]."""
     _need_gpu(q, cache, block_table, positions, seq_of_token)
     if q.dim() != 3 or q.stride(2) != 1 or q.stride(1) != q.shape[2]:
         raise KernelError("q must be [T, Hq, hd] with contiguous heads")
@@ -606,6 +609,14 @@ def paged_attention_simple(
         raise KernelError("a window holds at least the query's own key")
     out = torch.empty((n_tokens, n_q * hd), dtype=q.dtype, device=q.device)
     lib = _build.load("attention_simple")
+    if max_keys is None:
+        max_keys = int(positions.max()) + 1 if n_tokens else 1
+    if window is not None:
+        max_keys = min(max_keys, window)
+    max_keys = max(1, max_keys)
+    partial = None
+    if max_keys > lib.cwm_attention_simple_segment_keys():
+        partial = torch.empty(n_tokens * n_q * lib.cwm_attention_simple_max_segments() * (hd + 2), dtype=torch.float32, device=q.device)
     _check(
         lib,
         lib.cwm_attention_simple(
@@ -613,7 +624,8 @@ def paged_attention_simple(
             ctypes.c_int(_code(q.dtype)), _ptr(block_table), ctypes.c_int(block_table.shape[1]),
             _ptr(positions), _ptr(seq_of_token), ctypes.c_int(n_tokens), ctypes.c_int(n_q), ctypes.c_int(n_kv),
             ctypes.c_int(hd), ctypes.c_int(cache.shape[3] // hd), ctypes.c_int(cache.shape[0]),
-            ctypes.c_int(-1 if window is None else window - 1), ctypes.c_float(scale), _stream(),
+            ctypes.c_int(-1 if window is None else window - 1), ctypes.c_float(scale),
+            ctypes.c_int(max_keys), _ptr(partial), _stream(),
         ),
     )
     return out
@@ -759,7 +771,7 @@ def paged_attention(
     hd = q.shape[2]
     if q.is_cuda and mfma_attention_takes(q.dtype, hd, cache.shape[3] // hd):
         return paged_attention_mfma(q, cache, block_table, batch, window, scale)
-    return paged_attention_simple(q, cache, block_table, batch.positions, batch.seq_of_token, window, scale)
+    return paged_attention_simple(q, cache, block_table, batch.positions, batch.seq_of_token, window, scale, max_keys=batch.max_kv_len)
 
 
 # --------------------------------------------------------------------------- #
