@@ -72,52 +72,48 @@ def build_batch(
     (`CacheManager.extend`)."""
     if not portions:
         raise BatchError("a step needs at least one portion")
-    seen = set()
-    token_parts: List[np.ndarray] = []
-    position_parts: List[np.ndarray] = []
-    seq_parts: List[np.ndarray] = []
-    cu_q = [0]
-    kv_lens: List[int] = []
-    q_lens: List[int] = []
-    slots: List[int] = []
-    rows: List[int] = []
-    rids: List[Hashable] = []
-    for b, portion in enumerate(portions):
-        if portion.rid in seen:
-            raise BatchError(f"request {portion.rid!r} appears twice in one step")
-        seen.add(portion.rid)
-        if portion.rid not in manager:
-            raise BatchError(f"request {portion.rid!r} has not been admitted")
-        toks = np.asarray(portion.tokens, dtype=np.int64).reshape(-1)
-        n_new = toks.size
-        if n_new == 0:
-            raise BatchError(f"request {portion.rid!r} brings no token to this step")
-        n_old = manager.length(portion.rid)
-        if any(m > 0 for m in manager.pages_missing(portion.rid, n_new)):
-            raise BatchError(f"request {portion.rid!r}: pages for {n_new} more tokens have not been reserved")
-        bad = (toks < 0) | (toks >= vocab_size)
-        if bad.any():
-            raise BatchError(
-                f"request {portion.rid!r}: token id {int(toks[bad][0])} is outside the vocabulary of {vocab_size}"
-            )
-        base = cu_q[-1]
-        for w in portion.want:
-            if not 0 <= int(w) < n_new:
-                raise BatchError(f"request {portion.rid!r}: wanted place {w} is outside its {n_new} tokens")
-            rows.append(base + int(w))
-        token_parts.append(toks.astype(np.int32))
-        position_parts.append(np.arange(n_old, n_old + n_new, dtype=np.int32))
-        seq_parts.append(np.full(n_new, b, dtype=np.int32))
-        cu_q.append(base + n_new)
-        kv_lens.append(n_old + n_new)
-        q_lens.append(n_new)
-        slots.append(manager.slot(portion.rid))
-        rids.append(portion.rid)
-    tokens = np.concatenate(token_parts)
-    positions = np.concatenate(position_parts)
-    seq_of_token = np.concatenate(seq_parts)
-
     n_seqs = len(portions)
+    rids: List[Hashable] = [portion.rid for portion in portions]
+    if len(set(rids)) != n_seqs:
+        twice = next(r for r in rids if rids.count(r) > 1)
+        raise BatchError(f"request {twice!r} appears twice in one step")
+    for rid in rids:
+        if rid not in manager:
+            raise BatchError(f"request {rid!r} has not been admitted")
+    q_lens = [len(portion.tokens) for portion in portions]
+    for rid, n_new in zip(rids, q_lens):
+        if n_new == 0:
+            raise BatchError(f"request {rid!r} brings no token to this step")
+    old_lens = [manager.length(rid) for rid in rids]
+    for rid, n_new in zip(rids, q_lens):
+        if any(m > 0 for m in manager.pages_missing(rid, n_new)):
+            raise BatchError(f"request {rid!r}: pages for {n_new} more tokens have not been reserved")
+    kv_lens = [o + n for o, n in zip(old_lens, q_lens)]
+    slots = [manager.slot(rid) for rid in rids]
+    n_tokens = sum(q_lens)
+    # all vectors at once: a decode step of many requests is many portions of one token
+    q_arr = np.asarray(q_lens, dtype=np.int64)
+    cu = np.zeros(n_seqs + 1, dtype=np.int64)
+    np.cumsum(q_arr, out=cu[1:])
+    tokens = np.fromiter((t for portion in portions for t in portion.tokens), dtype=np.int64, count=n_tokens)
+    bad = (tokens < 0) | (tokens >= vocab_size)
+    if bad.any():
+        where = int(np.argmax(bad))
+        b = int(np.searchsorted(cu, where, side="right")) - 1
+        raise BatchError(f"request {rids[b]!r}: token id {int(tokens[where])} is outside the vocabulary of {vocab_size}")
+    seq_of_token = np.repeat(np.arange(n_seqs, dtype=np.int32), q_arr)
+    # position of a token: its place in the portion plus what the sequence held before
+    positions = (np.arange(n_tokens, dtype=np.int64) - np.repeat(cu[:-1] - np.asarray(old_lens, dtype=np.int64), q_arr)).astype(np.int32)
+    tokens = tokens.astype(np.int32)
+    rows: List[int] = []
+    for b, portion in enumerate(portions):
+        base = int(cu[b])
+        for w in portion.want:
+            if not 0 <= int(w) < q_lens[b]:
+                raise BatchError(f"request {portion.rid!r}: wanted place {w} is outside its {q_lens[b]} tokens")
+            rows.append(base + int(w))
+    cu_q = cu
+
     page_size = manager.page_size
     width = max(1, max((kv + page_size - 1) // page_size for kv in kv_lens))
     tables = []
