@@ -13,9 +13,10 @@ with random numbers instead of being computed (the weights are random too).
 
 `points` holds the workload that the baseline names: batches of 1, 8 and 64 requests with
 prompts of 1,024 random tokens and 256 new tokens each, through `Engine.step` (scheduler,
-step function and sampler, a host round trip per step); `decode_b<N>` is N times the number
-of steps in which all N requests decode, over the time of those steps; `decode_b<N>_ms` is the
-median of their times and `decode_b<N>_frac` the bytes such a step has to read over that
+step function and sampler; decode steps run in bursts of `sync_freq` = 10 with one host round
+trip a burst, as the reference's do); `decode_b<N>` is N times the number of steps in which all
+N requests decode, over the time of those steps; `decode_b<N>_ms` is the median of their times
+(a burst's time divided by its steps) and `decode_b<N>_frac` the bytes such a step has to read over that
 median and the HBM peak.  `decode_b8_ctx<C>` are decode steps of 8 requests at other context
 lengths through the step function, as the headline.
 """
@@ -335,7 +336,8 @@ def engine_point(model, batch, prompt_tokens, new_tokens, page, vocab):
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - start
         if engine.last_step_sequences == batch and engine.last_step_tokens == batch:
-            times.append(elapsed)
+            # a call runs `last_step_burst` decode steps back to back (sync_freq) and syncs with the host once
+            times.extend([elapsed / engine.last_step_burst] * engine.last_step_burst)
     assert finished == batch
     del engine
     torch.cuda.empty_cache()

@@ -39,7 +39,8 @@ class GenArgs:
     prefill_gb: float = 2  # memory kept free for activations when max_seq is negative
     gpu_gb: float = 74  # the reference's memory budget: ignored, free memory is measured
 
-    sync_freq: int = 10  # decode steps between host syncs in the reference: every step here
+    sync_freq: int = 10  # decode steps that run back to back, each fed by the tokens the one before sampled on the
+    # device, before tokens come to the host (whenever a step holds decoded tokens only and pages for all of them are free)
     handover_frequency: int = 0  # yield None every so many steps (0: never)
 
     def __post_init__(self) -> None:

@@ -67,9 +67,12 @@ def build_batch(
     manager: CacheManager,
     device: torch.device,
     vocab_size: int,
+    tokens_device: Optional[torch.Tensor] = None,
 ) -> StepBatch:
     """Descriptor for `portions`; the pages of their tokens must already be held
-    (`CacheManager.extend`)."""
+    (`CacheManager.extend`).  `tokens_device` (int32 [T] on the device) takes the place of the
+    portions' token ids, which then only count: a decode step whose tokens the step before has
+    sampled and which have not been to the host."""
     if not portions:
         raise BatchError("a step needs at least one portion")
     n_seqs = len(portions)
@@ -165,11 +168,14 @@ def build_batch(
     def seg(i: int) -> torch.Tensor:
         return dev[offsets[i] : offsets[i] + segments[i].size]
 
+    if tokens_device is not None:
+        if tokens_device.dtype != torch.int32 or tokens_device.numel() != tokens.size or not tokens_device.is_contiguous():
+            raise BatchError(f"tokens on the device must be a contiguous int32 [{tokens.size}] tensor")
     return StepBatch(
         n_tokens=int(tokens.size),
         n_seqs=n_seqs,
         n_logit_rows=len(rows),
-        tokens=seg(0),
+        tokens=seg(0) if tokens_device is None else tokens_device.reshape(-1),
         positions=seg(1),
         seq_of_token=seg(2),
         cu_q=seg(3),

@@ -150,12 +150,14 @@ class Engine:
         else:
             self.max_seq = args.max_seq if args.max_seq > 0 else max(sizes.values()) * args.cache_block
         # counters in the manner of the reference's throughput log (serve/fgserve.py:330-349)
-        self.n_steps = 0
+        self.n_steps = 0  # model steps
+        self.n_iterations = 0  # calls of step(): a burst of decode steps is one
         self.n_sequences = 0
         self.n_generated = 0
         self._reported = 0
         self.last_step_tokens = 0  # tokens and sequences that the latest step ran
         self.last_step_sequences = 0
+        self.last_step_burst = 1  # decode steps that the latest call of step() ran without a host sync between them
 
     # ---- construction ------------------------------------------------------------ #
     @classmethod
@@ -272,6 +274,7 @@ class Engine:
     def step(self) -> List[Packet]:
         """Schedule, run and sample one step; returns the requests it finished."""
         sched = self.scheduler
+        self.n_iterations += 1
         if self._profile_state != "inactive":
             self._profile_step()
         already = 0 if not sched.finished else len(sched.finished)
@@ -293,7 +296,14 @@ class Engine:
                 self.storage.zero_state(self.manager.slot(item.request.rid))
         self.last_step_sequences = len(batch)
         self.last_step_tokens = sum(item.count for item in batch)
-        if batch:
+        burst = 1
+        if batch and self.args.sync_freq > 1 and all(item.count == 1 and item.wants_logits for item in batch):
+            if not any(item.request.want_prompt_logprobs and len(item.request.prompt_logprobs) < len(item.request.prompt) - 1 for item in batch):
+                burst = sched.reserve_burst(batch, self.args.sync_freq)
+        self.last_step_burst = burst
+        if burst > 1:
+            self._decode_burst(batch, burst)
+        elif batch:
             logits = self.runner.step(sched.portions(batch))
             self.n_steps += 1
             # rows of `logits`: per entry its prompt places, then its sampling place
@@ -336,6 +346,40 @@ class Engine:
         # what has been handed back is not kept: a long-lived generate(q) would collect every request
         del sched.finished[:]
         return out
+
+    def _decode_burst(self, batch: List[Any], steps: int) -> None:
+        """`steps` decode steps of the same requests without a word from the host in between
+        (cwm/fastgen/generate.py:729-809): each step's tokens are sampled on the device and feed
+        the next step from there; tokens and log-probabilities come to the host once, at the end.
+        Pages for all the steps are reserved (`Scheduler.reserve_burst`)."""
+        from .batch import Portion
+
+        requests = [item.request for item in batch]
+        n = len(requests)
+        params = torch.tensor(
+            [[r.temperature for r in requests], [r.top_p for r in requests]]
+            + [[r.rng.next_uniform() if r.temperature > 0 else 0.0 for r in requests] for _ in range(steps)],
+            dtype=torch.float32,
+        )
+        if self.device.type == "cuda":
+            params = params.pin_memory()
+        params = params.to(self.device, non_blocking=True)
+        first = self.scheduler.portions(batch)
+        results = []
+        tokens_device = None
+        for k in range(steps):
+            portions = first if k == 0 else [Portion(rid=r.rid, tokens=[0], want=[0]) for r in requests]
+            logits = self.runner.step(portions, tokens_device)
+            tokens_device, logprob, sample_logprob = self.sampler.sample_on_device(logits, params[0], params[1], params[2 + k])
+            results.append((tokens_device, logprob, sample_logprob))
+        self.n_steps += steps
+        packed = torch.stack([torch.stack([t.to(torch.float64), a.to(torch.float64), b.to(torch.float64)]) for t, a, b in results]).cpu()
+        tokens = [[int(x) for x in packed[k, 0].tolist()] for k in range(steps)]
+        logprobs = [packed[k, 1].tolist() for k in range(steps)]
+        sample_logprobs = [packed[k, 2].tolist() for k in range(steps)]
+        before = sum(len(r.generated) for r in requests)
+        self.scheduler.burst_done(batch, tokens, self.stop_tokens, logprobs, sample_logprobs)
+        self.n_generated += sum(len(r.generated) for r in requests) - before
 
     # ---- the reference's generator interface ------------------------------------------ #
     def generate(self, q: "queue.Queue[Optional[Packet]]") -> Generator[Optional[Packet], None, None]:

@@ -49,12 +49,13 @@ class ModelRunner:
 
     # ---- the step ---------------------------------------------------------------- #
     @torch.inference_mode()
-    def step(self, portions: Sequence[Portion]) -> Optional[torch.Tensor]:
+    def step(self, portions: Sequence[Portion], tokens_device: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Run `portions` (pages already reserved with `CacheManager.extend`) and
         return logits [R, V], rows ordered by portion and then by `want`; None if no
         place is wanted.  Afterwards every request's length has grown by its portion
-        and window groups have given back the pages that fell out of reach."""
-        batch = build_batch(portions, self.manager, self.device, self.model.vocab_size)
+        and window groups have given back the pages that fell out of reach.  With
+        `tokens_device` the token ids come from that device tensor (see `build_batch`)."""
+        batch = build_batch(portions, self.manager, self.device, self.model.vocab_size, tokens_device)
         logits = self.model.forward(batch, self.storage)
         for portion in portions:
             self._report(self.manager.advance(portion.rid, len(portion.tokens)))

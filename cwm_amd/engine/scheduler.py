@@ -249,6 +249,56 @@ class Scheduler:
             return self.schedule()
         return batch
 
+    def reserve_burst(self, batch: Sequence[Scheduled], steps: int) -> int:
+        """`batch` holds one decoded token per request and its pages are reserved.  Reserve pages
+        for up to `steps` tokens each (the reference grows every lane to len + sync_freq before a
+        burst of decode steps, cwm/fastgen/generate.py:545-580), no further than any request may
+        grow; all or nothing: returns the steps reserved, 1 if the further pages are not there."""
+        steps = min([steps] + [item.request.max_len - len(item.request) for item in batch])
+        if steps <= 1:
+            return 1
+        # pages for `steps` tokens from each request's length on (the first token's are held already): do the
+        # pools have them, all requests together?
+        need = [0] * len(self.manager.groups)
+        for item in batch:
+            for g, missing in enumerate(self.manager.pages_missing(item.request.rid, steps)):
+                need[g] += missing
+        if any(n > free for n, free in zip(need, self.manager.free_pages())):
+            return 1
+        for item in batch:
+            if not self.manager.extend(item.request.rid, steps):
+                raise AssertionError("pages that were counted free are not there")
+        return steps
+
+    def burst_done(
+        self,
+        batch: Sequence[Scheduled],
+        tokens: Sequence[Sequence[int]],
+        stop_tokens: Set[int],
+        logprobs: Optional[Sequence[Sequence[float]]] = None,
+        sample_logprobs: Optional[Sequence[Sequence[float]]] = None,
+    ) -> None:
+        """`tokens[k][i]` is the token that step k of a burst sampled for the i-th request of
+        `batch`; step k + 1 has already run on it.  A request that stops inside the burst keeps
+        the tokens up to its stop token (cwm/fastgen/generate.py:681-727); what ran after it is
+        dropped with its pages."""
+        for i, item in enumerate(batch):
+            request = item.request
+            for k in range(len(tokens)):
+                request.cached += 1
+                token = int(tokens[k][i])
+                request.generated.append(token)
+                if logprobs is not None:
+                    request.logprobs.append(float(logprobs[k][i]))
+                if sample_logprobs is not None:
+                    request.sample_logprobs.append(float(sample_logprobs[k][i]))
+                if token in stop_tokens:
+                    self._finish(request, "stop")
+                    break
+                if len(request) >= request.max_len:
+                    self._finish(request, "length")
+                    break
+
     def portions(self, batch: Sequence[Scheduled]) -> List[Portion]:
         out = []
         for item in batch:

@@ -42,6 +42,14 @@ class Sampler:
     def __init__(self, device: torch.device) -> None:
         self.device = device
 
+    def sample_on_device(
+        self, logits: torch.Tensor, temperatures: torch.Tensor, top_ps: torch.Tensor, uniforms: torch.Tensor
+    ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        """The same with parameters and results on the device (float32 [R] each in; int32 tokens and
+        two float32 log-probabilities out): nothing waits for the host, so that the tokens can feed
+        the next step as they are."""
+        return ops.sample(logits, temperatures, top_ps, uniforms)
+
     def sample(
         self,
         logits: torch.Tensor,

@@ -258,3 +258,58 @@ def test_metrics_log_and_profile_window(tmp_path, monkeypatch):
     other = _engine(folder, monkeypatch)
     other.generate_tokens(prompts[:1], max_gen=2)
     assert len(path.read_text().splitlines()) == len(records)
+
+
+def test_decode_bursts_give_the_same_tokens_as_single_steps(tmp_path, monkeypatch):
+    """sync_freq decode steps run back to back, each fed by the tokens the one before sampled on
+    the device; the host sees tokens once a burst.  Same tokens as one step at a time, greedy and
+    sampled; a stop token inside a burst ends its request there and is kept; no request outgrows
+    its max_gen; a burst is not started when its pages are not free."""
+    from cwm_amd.engine import Engine, GenArgs, Packet
+
+    folder = models.make_folder(tmp_path, "tiny_b", seed=2, dtype="float32")
+    vocab = configs.get("tiny_b")["vocab_size"]
+    prompts = {f"p{i}": traces.random_tokens(70 + i, n, vocab) for i, n in enumerate([9, 30, 17])}
+
+    def run(sync_freq, stop=(), max_seq=1024, **kw):
+        cpu_ops.install(monkeypatch)
+        args = GenArgs(**{"use_sampling": True, "temperature": 0.8, "top_p": 0.9, "max_batch": 4, "max_seq": max_seq,
+                          "cache_block": 4, "max_prefill": 16, "sync_freq": sync_freq, "logprobs": True, **kw})
+        engine = Engine.from_folder(folder, args, dtype="float32", device="cpu", stop_tokens=stop, seed=5)
+        q = queue.Queue()
+        for i, (rid, toks) in enumerate(prompts.items()):
+            q.put(Packet(thread_id=rid, tokens=toks, max_gen=[23, 7, 12][i], temperature=0.0 if i == 2 else None))
+        q.put(None)
+        bursts = []
+        out = {}
+        for pkt in engine.generate(q):
+            bursts.append(engine.last_step_burst)
+            if pkt is not None:
+                out[pkt.thread_id] = pkt
+        engine.manager.check()
+        assert engine.manager.live_requests() == []
+        return out, bursts, engine
+
+    single, bursts1, _ = run(1)
+    assert set(bursts1) == {1}
+    many, bursts10, engine = run(10)
+    assert max(bursts10) > 1 and engine.n_steps > engine.n_iterations
+    for rid in prompts:
+        assert many[rid].tokens == single[rid].tokens
+        assert len(many[rid].tokens) == {"p0": 23, "p1": 7, "p2": 12}[rid]
+        assert max(abs(a - b) for a, b in zip(many[rid].logprobs, single[rid].logprobs)) < 1e-5
+        assert many[rid].sample_logprobs == pytest.approx(single[rid].sample_logprobs, abs=1e-5)
+    # a stop token in the middle of p0's tokens: the burst that contains it ends p0 there
+    stop = single["p0"].tokens[11]
+    cut = single["p0"].tokens.index(stop)
+    stopped, _, _ = run(10, stop=[stop])
+    assert stopped["p0"].tokens == single["p0"].tokens[: cut + 1] and stopped["p0"].finish_reason == "stop"
+    for rid in ("p1", "p2"):
+        want = single[rid].tokens
+        if stop in want:
+            want = want[: want.index(stop) + 1]
+        assert stopped[rid].tokens == want
+    # a cache with hardly a page to spare: bursts that do not fit are not started, tokens stay the same
+    tight, bursts_tight, _ = run(10, max_seq=96)
+    for rid in prompts:
+        assert tight[rid].tokens == single[rid].tokens
