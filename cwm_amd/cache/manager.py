@@ -23,18 +23,42 @@ from dataclasses import dataclass
 from typing import Dict, Hashable, List, Mapping, Optional, Sequence, Tuple, Union
 
 from ..parts.base import CacheSpec, PagedKVSpec, StateSpec
-from .pages import GroupTable, OutOfPages, PageAccountingError, PagePool, first_page_needed, pages_for
+from .pages import GroupTable, OutOfPages, PageAccountingError, PagePool, pages_for
 
 
 @dataclass
 class LayerGroup:
     """Cache slots whose layers keep the same span of keys: they share a pool and
-    block tables, and each has pages of its own in device memory."""
+    block tables, and each has pages of its own in device memory.  Which keys are
+    kept is the answer of `spec`, the need of the group's first slot."""
 
     index: int
-    window: Optional[int]
+    spec: PagedKVSpec
     cache_ids: List[int]
     pool: PagePool
+
+    @property
+    def window(self) -> Optional[int]:
+        return self.spec.window
+
+    def first_page_needed(self, length: int, page_size: int) -> int:
+        """Lowest logical page, pinned ones apart, that a query at position >= `length`
+        can still read."""
+        return self.spec.first_key_needed(length) // page_size
+
+    def pinned_pages(self, page_size: int) -> int:
+        """Logical pages at the start of a sequence that are never given back."""
+        return pages_for(self.spec.pinned_keys(), page_size)
+
+    def most_pages(self, length: int, step_tokens: int, page_size: int) -> int:
+        """Most pages that a request of `length` tokens holds of this group at any time
+        when a step brings at most `step_tokens` (a page of slack for where the span
+        starts inside a page)."""
+        need = pages_for(length, page_size)
+        span = self.spec.keys_kept(step_tokens)
+        if span is not None:
+            need = min(need, self.pinned_pages(page_size) + pages_for(span, page_size) + 1)
+        return need
 
 
 class _Request:
@@ -57,7 +81,8 @@ class CacheManager:
     ) -> None:
         """`specs[i]` is what cache slot i needs (a `PagedKVSpec`, a `StateSpec` or
         None).  `num_pages` is the pool size of every group, or a mapping from a
-        group's window (None for the keep-all group) to its pool size."""
+        group's `retention()` (for the built-in need its window, None for the keep-all
+        group) to its pool size."""
         if page_size <= 0:
             raise ValueError("page_size must be positive")
         if max_requests <= 0:
@@ -68,21 +93,22 @@ class CacheManager:
         self.groups: List[LayerGroup] = []
         self.group_of_cache: Dict[int, int] = {}
         self.state_caches: List[int] = []
-        by_window: Dict[Optional[int], LayerGroup] = {}
+        by_retention: Dict[Hashable, LayerGroup] = {}
         for cid, spec in enumerate(self.specs):
             if isinstance(spec, PagedKVSpec):
                 if spec.window is not None and spec.window < 1:
                     raise ValueError("a window holds at least one key")
-                grp = by_window.get(spec.window)
+                key = spec.retention()
+                grp = by_retention.get(key)
                 if grp is None:
                     if isinstance(num_pages, Mapping):
-                        if spec.window not in num_pages:
-                            raise ValueError(f"no pool size given for the group with window {spec.window}")
-                        n = num_pages[spec.window]
+                        if key not in num_pages:
+                            raise ValueError(f"no pool size given for the group that keeps {key!r}")
+                        n = num_pages[key]
                     else:
                         n = num_pages
-                    grp = LayerGroup(index=len(self.groups), window=spec.window, cache_ids=[], pool=PagePool(n))
-                    by_window[spec.window] = grp
+                    grp = LayerGroup(index=len(self.groups), spec=spec, cache_ids=[], pool=PagePool(n))
+                    by_retention[key] = grp
                     self.groups.append(grp)
                 grp.cache_ids.append(cid)
                 self.group_of_cache[cid] = grp.index
@@ -147,7 +173,8 @@ class CacheManager:
 
     def advance(self, rid: Hashable, n_new: int) -> List[List[int]]:
         """The step has written `n_new` tokens.  Returns, per group, the pages
-        given back because the window has passed them."""
+        given back because no later query reads them (the window has passed them, and
+        they are not pinned)."""
         req = self._requests[rid]
         new_len = req.length + n_new
         if any(len(req.tables[g.index].pages) < pages_for(new_len, self.page_size) for g in self.groups):
@@ -157,8 +184,8 @@ class CacheManager:
         for g in self.groups:
             table = req.tables[g.index]
             gone: List[int] = []
-            first = first_page_needed(new_len, g.window, self.page_size)
-            for lp in range(table.first_held, min(first, len(table.pages))):
+            first = g.first_page_needed(new_len, self.page_size)
+            for lp in range(max(table.first_held, g.pinned_pages(self.page_size)), min(first, len(table.pages))):
                 page = table.pages[lp]
                 if page >= 0:
                     g.pool.give(page)

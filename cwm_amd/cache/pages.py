@@ -64,7 +64,7 @@ class GroupTable:
 
     def __init__(self) -> None:
         self.pages: List[int] = []
-        self.first_held = 0  # every logical page below this index has been given back
+        self.first_held = 0  # every logical page below this index has been given back, pinned ones apart
 
     def held(self) -> List[int]:
         return [p for p in self.pages if p >= 0]

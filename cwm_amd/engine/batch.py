@@ -16,7 +16,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager
-from ..cache.pages import first_page_needed, pages_for
+from ..cache.pages import pages_for
 
 
 @dataclass
@@ -130,9 +130,9 @@ def build_batch(
             tbl[b, :n] = pages[:n]
         # every page that this step's queries can read, or that its tokens are written to, is held
         first_page = np.asarray(
-            [first_page_needed(kv - q, g.window, page_size) for kv, q in zip(kv_lens, q_lens)], dtype=np.int64
+            [g.first_page_needed(kv - q, page_size) for kv, q in zip(kv_lens, q_lens)], dtype=np.int64
         )[:, None]
-        needed = (columns >= first_page) & (columns < last_page)
+        needed = ((columns >= first_page) | (columns < g.pinned_pages(page_size))) & (columns < last_page)
         bad = needed & ((tbl < 0) | (tbl >= g.pool.num_pages))
         if bad.any():
             b = int(np.argmax(bad.any(axis=1)))

@@ -17,7 +17,7 @@ from __future__ import annotations
 import os
 import queue
 import time
-from typing import Any, Dict, Generator, Iterable, List, Optional, Sequence, Union
+from typing import Any, Dict, Generator, Hashable, Iterable, List, Optional, Sequence, Union
 
 import torch
 
@@ -38,9 +38,9 @@ def pool_sizes(
     args: GenArgs,
     device: torch.device,
     free_bytes: Optional[int] = None,
-) -> Dict[Optional[int], int]:
-    """Pages of every layer group (keyed by the group's window, None for the group that keeps
-    all keys).
+) -> Dict[Hashable, int]:
+    """Pages of every layer group, keyed by what the group's cache need answers to `retention()`
+    (its window; None for the group that keeps all keys).
 
     With `max_seq` given, the keep-all group holds that many tokens
     (cwm/fastgen/generate.py:245-251) and a group with window W the same, or less if
@@ -60,22 +60,27 @@ def pool_sizes(
     """
     page = args.cache_block
     esize = 4 if model.runtime.act_dtype == torch.float32 else 2
-    per_page: Dict[Optional[int], int] = {}
+    per_page: Dict[Hashable, int] = {}
+    kept: Dict[Hashable, Optional[int]] = {}  # most tokens one request holds of a group; None: all
     for spec in model.cache_specs:
         if isinstance(spec, PagedKVSpec):
-            per_page[spec.window] = per_page.get(spec.window, 0) + 2 * spec.n_kv_heads * spec.head_dim * page * esize
+            key = spec.retention()
+            per_page[key] = per_page.get(key, 0) + 2 * spec.n_kv_heads * spec.head_dim * page * esize
+            span = spec.keys_kept(args.max_prefill)
+            kept[key] = None if span is None else spec.pinned_keys() + span
     if not per_page:
         return {}
+    keep_all = [key for key in per_page if kept[key] is None]
 
-    def request_cap(window: int) -> int:
-        """Most pages that `max_batch` requests can hold of a window group."""
-        return args.max_batch * ((window - 1 + args.max_prefill + page - 1) // page + 2)
+    def request_cap(tokens: int) -> int:
+        """Most pages that `max_batch` requests can hold of a group that keeps `tokens` of each."""
+        return args.max_batch * ((tokens + page - 1) // page + 2)
 
-    sizes: Dict[Optional[int], int] = {}
+    sizes: Dict[Hashable, int] = {}
     if args.max_seq > 0:
         cap_pages = (args.max_seq + page - 1) // page
-        for w in per_page:
-            sizes[w] = max(1, cap_pages if w is None else min(request_cap(w), cap_pages))
+        for key in per_page:
+            sizes[key] = max(1, cap_pages if kept[key] is None else min(request_cap(kept[key]), cap_pages))
         return sizes
 
     if free_bytes is None:
@@ -86,22 +91,24 @@ def pool_sizes(
     budget = int(0.9 * (free_bytes - int(args.prefill_gb * 1e9)))
     expected = args.expected_seq if args.expected_seq > 0 else (model.plan.max_positions or 0)
     # pages that one expected request holds of each group
-    share: Dict[Optional[int], int] = {}
-    for w in per_page:
+    share: Dict[Hashable, int] = {}
+    for key in per_page:
         if expected <= 0:
-            share[w] = 1
+            share[key] = 1
         else:
-            tokens = expected if w is None else min(expected, w - 1 + args.max_prefill)
-            share[w] = (tokens + page - 1) // page + 1
-    per_request = sum(share[w] * per_page[w] for w in per_page)
+            tokens = expected if kept[key] is None else min(expected, kept[key])
+            share[key] = (tokens + page - 1) // page + 1
+    per_request = sum(share[key] * per_page[key] for key in per_page)
     requests = budget / per_request if budget > 0 else 0.0
-    for w in per_page:
-        sizes[w] = int(requests * share[w])
-        if w is not None and sizes[w] > request_cap(w):
-            sizes[w] = request_cap(w)
-    if None in per_page:  # what the caps saved
-        rest = budget - sum(sizes[w] * per_page[w] for w in per_page if w is not None)
-        sizes[None] = max(sizes[None], rest // per_page[None])
+    for key in per_page:
+        sizes[key] = int(requests * share[key])
+        if kept[key] is not None and sizes[key] > request_cap(kept[key]):
+            sizes[key] = request_cap(kept[key])
+    if keep_all:  # what the caps saved
+        rest = budget - sum(sizes[key] * per_page[key] for key in per_page if kept[key] is not None)
+        per_token = sum(per_page[key] for key in keep_all)
+        for key in keep_all:
+            sizes[key] = max(sizes[key], rest // per_token)
     smallest = min(sizes.values())
     if smallest < 1:
         raise MemoryError(

@@ -142,10 +142,7 @@ class Scheduler:
         total = max(len(request), min(len(request) + self.headroom, request.max_len))
         page = self.manager.page_size
         for group, free in zip(self.manager.groups, self.manager.free_pages()):
-            need = pages_for(total, page)
-            if group.window is not None:
-                need = min(need, pages_for(group.window - 1 + self.max_tokens_per_step, page) + 1)
-            if need > free:
+            if group.most_pages(total, self.max_tokens_per_step, page) > free:
                 return False
         return True
 

@@ -16,7 +16,7 @@ Kinds of part and their registries (name -> class):
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Callable, Dict, List, Mapping, Optional, Tuple, Union
+from typing import Any, Callable, Dict, Hashable, List, Mapping, Optional, Tuple, Union
 
 import torch
 
@@ -47,6 +47,33 @@ class PagedKVSpec:
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+
+    # What the cache manager asks.  A mixer with another rule (keys pinned at the start
+    # of a sequence beside a window, say) passes a subclass that answers differently;
+    # the manager, the scheduler and the pool sizes know these four methods only.
+    def retention(self) -> Hashable:
+        """Cache slots whose values are equal keep the same keys: they share a pool and
+        block tables.  It is also the key under which a pool size is given."""
+        return self.window
+
+    def first_key_needed(self, length: int) -> int:
+        """Lowest position, pinned keys apart, that a query at position >= `length` can
+        still read.  A layer with window W lets the query at position p read keys
+        p-(W-1)..p (cwm/model/transformer.py:253-270)."""
+        if self.window is None:
+            return 0
+        return max(0, length - (self.window - 1))
+
+    def pinned_keys(self) -> int:
+        """Keys at the start of a sequence that every later query reads."""
+        return 0
+
+    def keys_kept(self, step_tokens: int) -> Optional[int]:
+        """Most keys, pinned ones apart, that a request holds at any time when a step
+        brings at most `step_tokens`; None if all are kept."""
+        if self.window is None:
+            return None
+        return self.window - 1 + step_tokens
 
 
 @dataclass(frozen=True)

@@ -5,6 +5,7 @@ than the window needs; reservation is all-or-nothing."""
 import random
 
 import pytest
+import torch
 
 from cwm_amd.cache import CacheManager, OutOfPages, PageAccountingError, PagePool, first_page_needed
 from cwm_amd.parts import PagedKVSpec, StateSpec
@@ -136,3 +137,59 @@ def test_random_orders_keep_the_accounts(seed):
     assert m.free_pages() == [g.pool.num_pages for g in m.groups]
     # pages were used again by other owners
     assert any(len(owners) > 1 for pages in handed.values() for owners in pages.values())
+
+
+def test_another_retention_rule_needs_no_change_to_the_manager():
+    """A cache need defined here, outside the framework: the first `sinks` keys are read by
+    every query, beside a window.  The manager keeps their pages, gives back what lies
+    between them and the window, groups the slot apart from a plain window of the same
+    length, and the scheduler's and the step's questions are answered by the same methods."""
+    from dataclasses import dataclass
+
+    from cwm_amd.engine.batch import BatchError, Portion, build_batch
+
+    @dataclass(frozen=True)
+    class PinnedStartSpec(PagedKVSpec):
+        sinks: int = 0
+
+        def retention(self):
+            return ("pinned start", self.sinks, self.window)
+
+        def pinned_keys(self):
+            return self.sinks
+
+    page = 4
+    specs_ = [
+        PinnedStartSpec(n_kv_heads=1, head_dim=16, window=8, sinks=5),
+        PagedKVSpec(n_kv_heads=1, head_dim=16, window=8),
+        PinnedStartSpec(n_kv_heads=1, head_dim=16, window=8, sinks=5),
+    ]
+    m = CacheManager(specs_, page_size=page, num_pages={("pinned start", 5, 8): 12, 8: 12}, max_requests=2)
+    assert [g.cache_ids for g in m.groups] == [[0, 2], [1]]
+    pinned, plain = m.groups
+    assert pinned.pinned_pages(page) == 2 and plain.pinned_pages(page) == 0
+    # a request of 1,000 tokens with steps of 6: 2 pinned pages + ceil((7 + 6) / 4) + 1 of slack
+    assert pinned.most_pages(1000, 6, page) == 2 + 4 + 1
+    assert plain.most_pages(1000, 6, page) == 4 + 1
+    assert pinned.most_pages(9, 6, page) == 3
+
+    m.admit("a")
+    for _ in range(10):
+        assert m.extend("a", 3)
+        m.advance("a", 3)
+        m.check()
+    # 30 tokens: the window's first key is 23, in page 5; pages 0 and 1 hold the pinned keys
+    assert [p >= 0 for p in m.table(pinned.index, "a")] == [True, True, False, False, False, True, True, True]
+    assert [p >= 0 for p in m.table(plain.index, "a")] == [False, False, False, False, False, True, True, True]
+    assert m.free_pages() == [12 - 5, 12 - 3]
+
+    # the step's check of the tables asks for the pinned pages too
+    assert m.extend("a", 1)
+    build_batch([Portion("a", [1], [0])], m, torch.device("cpu"), vocab_size=10)
+    m.table(pinned.index, "a")[1] = -1
+    with pytest.raises(BatchError, match="holds no page"):
+        build_batch([Portion("a", [1], [0])], m, torch.device("cpu"), vocab_size=10)
+    m.table(pinned.index, "a")[1] = 1
+    m.release("a")
+    m.check()
+    assert m.free_pages() == [12, 12]
