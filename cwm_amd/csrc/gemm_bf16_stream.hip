@@ -39,8 +39,12 @@ union Frag8 {
 
 // block shapes: {tiles of A, wavefronts, steps of 32 along K in half a W tile}; a wavefront
 // holds 2 * half steps of each of its tiles of A in registers
+#ifndef ST1_WAVES
 #define ST1_WAVES 16
+#endif
+#ifndef ST1_HALF
 #define ST1_HALF 6
+#endif
 #ifndef ST4_WAVES
 #define ST4_WAVES 16
 #endif

@@ -187,3 +187,75 @@ def test_empty_prompt_is_refused():
     manager = CacheManager([PagedKVSpec(1, 8, None)], 4, 8, 2)
     with pytest.raises(ValueError):
         Scheduler(manager, 2, 8).add(Request(rid=0, prompt=[], max_len=4))
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_workloads_give_the_tokens_of_an_undisturbed_run(seed):
+    """Random prompts, arrival times, pools, page sizes, windows, budgets, headroom and decode
+    bursts: whatever is preempted, recomputed or cut, a request's tokens are those it would
+    get alone, and the books balance after every step."""
+    import random
+
+    rng = random.Random(seed)
+    page_size = rng.choice([1, 2, 4, 8, 16])
+    max_batch = rng.choice([1, 2, 4, 6])
+    budget = rng.choice([2, 5, 16, 64])
+    window = rng.choice([None, 3, 8, 20])
+    headroom = rng.choice([0, 0, 4, 128])
+    burst = rng.choice([1, 1, 3, 10])
+    stop = {rng.randrange(VOCAB)} if rng.random() < 0.5 else set()
+    n_requests = rng.randrange(1, 12)
+    todo = []
+    for i in range(n_requests):
+        prompt = [rng.randrange(VOCAB) for _ in range(rng.choice([1, 2, 7, 19, 40, 90]))]
+        todo.append((rng.randrange(0, 30), Request(rid=i, prompt=prompt, max_len=len(prompt) + rng.choice([1, 2, 9, 33, 80]))))
+    longest = max(r.max_len for _, r in todo)
+    # from a pool that preempts all the time to one that never does; always enough for the longest request alone
+    pages_alone = -(-longest // page_size) + 1
+    num_pages = pages_alone + rng.choice([0, 1, 3, 5, 12, 40, 400])
+    specs = [PagedKVSpec(1, 8, None), PagedKVSpec(1, 8, window)]
+    manager = CacheManager(specs, page_size, num_pages, max_batch)
+    sched = Scheduler(manager, max_batch, budget, headroom=headroom)
+    todo.sort(key=lambda pair: pair[0])
+    steps = 0
+    while todo or sched.has_work():
+        while todo and todo[0][0] <= steps:
+            sched.add(todo.pop(0)[1])
+        steps += 1
+        assert steps < 20000, "the scheduler does not finish"
+        if not sched.has_work():
+            continue
+        batch = sched.schedule()
+        assert sum(item.count for item in batch) <= budget
+        assert len(sched.running) <= max_batch
+        decode_only = bool(batch) and all(item.count == 1 and item.wants_logits and item.request.generated for item in batch)
+        n = sched.reserve_burst(batch, burst) if decode_only and burst > 1 else 1
+        if n > 1:
+            rows = []
+            sofar = [item.request.all_tokens() for item in batch]
+            for _ in range(n):
+                for item in batch:
+                    manager.advance(item.request.rid, 1)
+                row = [next_token(toks) for toks in sofar]
+                for toks, t in zip(sofar, row):
+                    toks.append(t)
+                rows.append(row)
+            sched.burst_done(batch, rows, stop)
+        else:
+            toks = []
+            for item, portion in zip(batch, sched.portions(batch)):
+                assert portion.tokens == item.request.all_tokens()[item.start : item.start + item.count]
+                assert item.start == manager.length(item.request.rid) == item.request.cached
+                manager.advance(item.request.rid, item.count)
+                if item.wants_logits:
+                    toks.append(next_token(item.request.all_tokens()))
+            sched.step_done(batch, toks, stop)
+        manager.check()
+    assert manager.live_requests() == []
+    assert manager.free_pages() == [g.pool.num_pages for g in manager.groups]
+    done = {r.rid: r for r in sched.finished}
+    assert sorted(done) == list(range(n_requests))
+    for r in done.values():
+        want = expected(r.prompt, r.max_len - len(r.prompt), stop)
+        assert r.generated == want, (r.rid, r.finish_reason)
+        assert r.finish_reason == ("stop" if want[-1] in stop else "length")
