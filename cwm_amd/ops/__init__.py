@@ -192,6 +192,11 @@ def gate_up_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
     )
     if fused:
         return gemm_bf16_stream(x, weight, bias, torch.bfloat16, glu=True)
+    if (
+        grouped and x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+        and STREAM_FUSED_ROWS < x.shape[0] <= TILE_ROWS and _tile_takes(x, weight)
+    ):
+        return gemm_bf16_tile(x, weight, bias, torch.bfloat16, glu=True)
     return silu_mul(linear(x, weight, bias, partials_ok=True), out_dtype=x.dtype, grouped=grouped)
 
 
@@ -473,6 +478,107 @@ def sum_partials(partials: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor
     return out
 
 
+TILE_MAX_ROWS = 512
+_tile_slabs: dict = {}  # (rows, columns, K, blocks) -> slabs of partial results
+
+
+def _tile_takes(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    k, n = x.shape[1], weight.shape[0]
+    return (
+        x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+        and k % 64 == 0 and n % 16 == 0 and 0 < x.shape[0] <= TILE_MAX_ROWS
+        and x.stride(-1) == 1 and weight.stride(-1) == 1
+        and (x.shape[0] <= 1 or x.stride(0) % 8 == 0) and (n <= 1 or weight.stride(0) % 8 == 0)
+        and max(x.stride(0), weight.stride(0)) < (1 << 22)
+        and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
+    )
+
+
+def gemm_bf16_tile(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    out_dtype: Optional[torch.dtype] = None,
+    partials_ok: bool = False,
+    glu: bool = False,
+    units: Optional[int] = None,
+) -> torch.Tensor:
+    """bfloat16 x [M <= 512, K] @ weight[N, K]^T with float32 sums: persistent blocks whose tiles
+    of 64 or 128 rows reach LDS by direct loads and that share the work by steps of K.  Returns
+    [M, N]; with `partials_ok` it may return float32 partial sums [P, M, N] for the caller to add.
+    `glu`: the weight's rows are gate and up rows in alternating groups of 8 and the result is
+    silu(gate) * up, [M, N / 2] (in the kernel where a block owns whole tiles, else after it).
+    `units` (tests) stands in for the number of compute units."""
+    _need_gpu(x, weight, bias)
+    if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1] or not _tile_takes(x, weight):
+        raise KernelError(
+            f"the tiled product takes bfloat16 x [0 < M <= {TILE_MAX_ROWS}, K] and weight [N, K] with K a multiple of 64, N of "
+            f"16 and 16-byte aligned rows; got {tuple(x.shape)} {x.dtype} and {tuple(weight.shape)} {weight.dtype}"
+        )
+    m, k = x.shape
+    n = weight.shape[0]
+    if bias is not None and (bias.shape != (n,) or not bias.is_contiguous()):
+        raise KernelError(f"gemm: bias {tuple(bias.shape)} does not fit {n} outputs")
+    out_dtype = out_dtype or torch.bfloat16
+    lib = _build.load("gemm_bf16_tile")
+    units = units or _compute_units(x.device)
+    slabs = _tile_slabs.get((m, n, k, units))
+    if slabs is None:
+        slabs = _tile_slabs[(m, n, k, units)] = int(lib.cwm_gemm_bf16_tile_slabs(m, n, k, units))
+        if slabs < 1:
+            raise KernelError(f"the tiled product has no cut for M={m} N={n} K={k}")
+    fused_glu = glu and slabs == 1 and bias is None
+    if fused_glu:
+        out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
+    elif slabs == 1:
+        out = torch.empty((m, n), dtype=torch.float32 if bias is not None else (torch.bfloat16 if glu else out_dtype), device=x.device)
+    else:
+        out = torch.empty((slabs, m, n), dtype=torch.float32, device=x.device)
+    _check(
+        lib,
+        lib.cwm_gemm_bf16_tile(
+            _ptr(x), ctypes.c_long(x.stride(0) if m > 1 else k), _ptr(weight), ctypes.c_long(weight.stride(0) if n > 1 else k),
+            _ptr(out), ctypes.c_int(_code(out.dtype)), ctypes.c_long(out.shape[-1]), ctypes.c_long(m * n),
+            ctypes.c_int(m), ctypes.c_int(n), ctypes.c_int(k), ctypes.c_int(units), ctypes.c_int(slabs), ctypes.c_int(int(fused_glu)),
+            _stream(),
+        ),
+    )
+    if fused_glu:
+        return out
+    if bias is not None:  # not in the kernel; no model of this architecture has one on a product of this size
+        if out.dim() == 3:
+            out[0] += bias.float()
+        else:
+            out = out + bias.float()
+    if glu:
+        return silu_mul(out if out.dim() == 3 else out.to(torch.bfloat16), out_dtype=torch.bfloat16, grouped=True)
+    if out.dim() == 3 and not partials_ok:
+        return sum_partials(out, out_dtype)
+    return out if out.dim() == 3 or out.dtype == out_dtype else out.to(out_dtype)
+
+
+STREAM_FUSED_ROWS = 16  # rows up to which the streaming product keeps x in registers and has every epilogue
+TILE_ROWS = 128  # rows up to which the tiled product reads W once
+TILE_ROWS_SHARED = 256  # rows up to which it still beats the library where blocks share tiles (a narrow result)
+
+
+def _tile_wins(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether the tiled product takes this product and is the fastest for it (measured on the 32B
+    shape's matrices: above 128 rows W is read once per 128 rows, which the library beats on wide results)."""
+    m = x.shape[0]
+    if m > TILE_ROWS_SHARED or not _tile_takes(x, weight):
+        return False
+    if m <= TILE_ROWS:
+        return True
+    lib = _build.load("gemm_bf16_tile")
+    units = _compute_units(x.device)
+    key = (m, weight.shape[0], x.shape[1], units)
+    slabs = _tile_slabs.get(key)
+    if slabs is None:
+        slabs = _tile_slabs[key] = int(lib.cwm_gemm_bf16_tile_slabs(*key))
+    return slabs > 1
+
+
 def _stream_takes(x: torch.Tensor, weight: torch.Tensor) -> bool:
     k = x.shape[1]
     return (
@@ -493,16 +599,20 @@ def gemm_bf16(
 ) -> torch.Tensor:
     """bfloat16 x [M, K] @ bfloat16 weight[N, K]^T, float32 accumulation.
 
-    Up to 64 rows: the hand-written persistent weight-streaming kernel.  More rows:
-    the library product (hipBLASLt through torch), as the reference calls a library
-    here, with a bfloat16 or a float32 result.  Row lengths that are no multiple of 8
-    go to the float32 kernel, which takes any size.
+    Up to 16 rows: the hand-written persistent weight-streaming kernel, x in registers.
+    Up to 128 rows (256 for a narrow result): the hand-written tiled kernel, x and W
+    through LDS (it needs K % 64 == 0 and N % 16 == 0; other sizes of up to 64 rows stream).
+    More rows: the library product (hipBLASLt through torch), as the reference calls a
+    library here, with a bfloat16 or a float32 result.  Row lengths that are no multiple
+    of 8 go to the float32 kernel, which takes any size.
     """
     _need_gpu(x, weight, bias)
     out_dtype = out_dtype or torch.bfloat16
     m = x.shape[0]
     if not _stream_takes(x, weight):
         return gemm_f32(x, weight, bias, out_dtype)
+    if m > STREAM_FUSED_ROWS and _tile_wins(x, weight):
+        return gemm_bf16_tile(x, weight, bias, out_dtype, partials_ok)
     if m <= STREAM_MAX_ROWS:
         return gemm_bf16_stream(x, weight, bias, out_dtype, partials_ok)
     if out_dtype == torch.float32:

@@ -53,6 +53,7 @@ SOURCES: Dict[str, Tuple[Mapping[str, int], ...]] = {
     "gemm_f32_stream": ({},),
     "sampling": ({},),
     "gemm_bf16_stream": ({},),
+    "gemm_bf16_tile": ({},),
     "attention_mfma": tuple({"HEAD_DIM": hd} for hd in (16, 32, 48, 64, 80, 96, 128, 256)),
 }
 

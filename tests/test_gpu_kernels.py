@@ -811,7 +811,7 @@ def test_gemm_bf16_stream(out_dtype, m, n, k):
     # views with a wider row stride (as the q/k/v and gate/up products are used)
     wide = torch.zeros((m, k + 24), dtype=torch.bfloat16)
     wide[:, 8 : 8 + k] = a
-    got2 = ops.gemm_bf16(wide.to(DEV)[:, 8 : 8 + k], w.to(DEV), b.to(DEV), out_dtype).cpu()
+    got2 = ops.gemm_bf16_stream(wide.to(DEV)[:, 8 : 8 + k], w.to(DEV), b.to(DEV), out_dtype).cpu()
     assert torch.equal(got2, got)
 
 
@@ -868,3 +868,85 @@ def test_qkv_rope_write_fused_equals_separate(n_q, n_kv, hd, page_size, dim, bia
     assert torch.equal(fused, qkv)
     assert torch.equal(caches[0], caches[1])
     assert caches[0].abs().sum() > 0
+
+
+@pytest.mark.parametrize(
+    "m,n,k,units",
+    [
+        (17, 16, 64, 4), (64, 208, 192, 3), (40, 1072, 256, 7), (65, 1072, 256, 7), (128, 5376, 512, 16), (100, 6144, 1024, None),
+        (200, 512, 128, 5), (256, 3072, 640, None), (33, 128256, 64, None), (64, 8192, 6144, None), (129, 96, 64, 2), (512, 192, 128, 3),
+    ],
+)
+def test_gemm_bf16_tile(m, n, k, units):
+    """The tiled product: whole tiles and tiles shared between blocks, against float64; `units`
+    stands in for the number of blocks that run at once, so that few blocks cut small products
+    the way 256 cut large ones."""
+    from cwm_amd import ops
+
+    a = rnd((m, k), torch.bfloat16, 6)
+    w = rnd((n, k), torch.bfloat16, 7, 0.05)
+    want = a.double() @ w.double().T
+    scale = float(want.abs().max())
+    limit = 1e-5 * scale * (1 + k / 512)
+    ad, wd = a.to(DEV), w.to(DEV)
+    # memory that the next result is likely to be given, full of NaN: what the kernel does not write shows
+    junk = torch.full((8, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    del junk
+    parts = ops.gemm_bf16_tile(ad, wd, None, torch.float32, partials_ok=True, units=units).cpu()
+    assert parts.dtype == torch.float32
+    total = parts.double().sum(0) if parts.dim() == 3 else parts.double()
+    assert (total - want).abs().max() <= limit
+    got = ops.gemm_bf16_tile(ad, wd, None, torch.float32, units=units).cpu()
+    assert got.shape == (m, n) and (got.double() - want).abs().max() <= limit
+    got_bf = ops.gemm_bf16_tile(ad, wd, None, torch.bfloat16, units=units).cpu()
+    assert got_bf.dtype == torch.bfloat16
+    torch.testing.assert_close(got_bf.double(), want, rtol=1e-2, atol=1e-2 * scale)
+    # a row's result does not depend on the other rows, among calls of one block height
+    fewer = m - 1 if m > 65 and (m - 1 + 127) // 128 == (m + 127) // 128 else (17 if 17 < m <= 64 else m)
+    if fewer != m:
+        one = ops.gemm_bf16_tile(ad[m - fewer :].contiguous(), wd, None, torch.float32, units=units).cpu()
+        assert torch.equal(one[-1], got[m - 1])
+    # a bias is added after the kernel
+    b = rnd((n,), torch.bfloat16, 8, 2.0)
+    got_b = ops.gemm_bf16_tile(ad, wd, b.to(DEV), torch.float32, units=units).cpu()
+    assert (got_b.double() - want - b.double()).abs().max() <= limit + 1e-6 * float(b.abs().max())
+    # views with a wider row stride
+    wide = torch.zeros((m, k + 24), dtype=torch.bfloat16)
+    wide[:, 8 : 8 + k] = a
+    assert torch.equal(ops.gemm_bf16_tile(wide.to(DEV)[:, 8 : 8 + k], wd, None, torch.float32, units=units).cpu(), got)
+
+
+@pytest.mark.parametrize("m,f,k,units", [(17, 48, 64, 1), (64, 21504 // 8, 6144 // 4, 16), (128, 1000, 192, 8), (100, 296, 128, 2), (30, 8, 64, 1)])
+def test_gemm_bf16_tile_gated_epilogue(m, f, k, units):
+    """The tiled product with silu(gate) * up in its epilogue against the product followed by the
+    activation kernel (the same bits), whichever cut the sizes get, and against float64."""
+    from cwm_amd import ops
+
+    x = rnd((m, k), torch.bfloat16, 1)
+    wg, wu = rnd((f, k), torch.bfloat16, 2, 0.2), rnd((f, k), torch.bfloat16, 3, 0.2)
+    w = torch.stack([wg.reshape(f // 8, 8, k), wu.reshape(f // 8, 8, k)], dim=1).reshape(2 * f, k).contiguous()
+    fused = ops.gemm_bf16_tile(x.to(DEV), w.to(DEV), None, torch.bfloat16, glu=True, units=units)
+    assert fused.shape == (m, f) and fused.dtype == torch.bfloat16
+    two_steps = ops.silu_mul(ops.gemm_bf16_tile(x.to(DEV), w.to(DEV), None, torch.bfloat16, units=units), grouped=True)
+    assert torch.equal(fused, two_steps)
+    g = x.double() @ wg.double().T
+    u = x.double() @ wu.double().T
+    want = g * torch.sigmoid(g) * u
+    torch.testing.assert_close(fused.cpu().double(), want, rtol=3e-2, atol=3e-2 * float(want.abs().max()))
+
+
+def test_products_of_17_to_128_rows_take_the_tiled_kernel():
+    """`linear` and `gate_up_silu` route the sizes the tiled kernel takes to it, and the others as before."""
+    from cwm_amd import ops
+
+    x = rnd((40, 128), torch.bfloat16, 1).to(DEV)
+    w = rnd((208, 128), torch.bfloat16, 2, 0.1).to(DEV)
+    assert torch.equal(ops.linear(x, w), ops.gemm_bf16_tile(x, w))
+    assert torch.equal(ops.gate_up_silu(x, w, None, True), ops.gemm_bf16_tile(x, w, glu=True))
+    odd = rnd((208, 120), torch.bfloat16, 3, 0.1).to(DEV)  # K no multiple of 64
+    xo = rnd((40, 120), torch.bfloat16, 4).to(DEV)
+    assert torch.equal(ops.linear(xo, odd), ops.gemm_bf16_stream(xo, odd))
+    with pytest.raises(ops.KernelError, match="tiled product takes"):
+        ops.gemm_bf16_tile(xo, odd)
+    x16 = x[:16].contiguous()
+    assert torch.equal(ops.linear(x16, w), ops.gemm_bf16_stream(x16, w))
