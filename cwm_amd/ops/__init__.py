@@ -457,13 +457,62 @@ def qkv_rope_write(
             x, weight, bias, torch.bfloat16,
             rope=(positions, seq_of_token, inv_freq, cache, block_table, n_q_heads, n_kv_heads, head_dim),
         )
-    qkv = linear(x, weight, bias)
+    qkv = linear(x, weight, bias, partials_ok=True)
+    if qkv.dim() == 3:
+        # partial sums of a split K: added by the rotation kernel where it can, else by a kernel of their own
+        if x.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and head_dim % 8 == 0 and head_dim <= 256:
+            return rope_kv_write_partials(qkv, n_q_heads, n_kv_heads, head_dim, positions, inv_freq, cache, block_table, seq_of_token)
+        qkv = sum_partials(qkv, x.dtype)
     q_out, kv_out = n_q_heads * head_dim, n_kv_heads * head_dim
     q = qkv[:, :q_out].unflatten(1, (n_q_heads, head_dim))
     k = qkv[:, q_out : q_out + kv_out].unflatten(1, (n_kv_heads, head_dim))
     v = qkv[:, q_out + kv_out :].unflatten(1, (n_kv_heads, head_dim))
     rope_kv_write(q, k, v, positions, inv_freq, cache, block_table, seq_of_token)
     return qkv
+
+
+def rope_kv_write_partials(
+    partials: torch.Tensor,
+    n_q_heads: int,
+    n_kv_heads: int,
+    head_dim: int,
+    positions: torch.Tensor,
+    inv_freq: Optional[torch.Tensor],
+    cache: torch.Tensor,
+    block_table: torch.Tensor,
+    seq_of_token: torch.Tensor,
+) -> torch.Tensor:
+    """`rope_kv_write` from the float32 partial sums [P, T, (Hq + 2 Hkv) * hd] of the joined q/k/v
+    projection: they are added in order and rounded to bfloat16 (the bits `sum_partials` gives), q
+    and k are rotated, k and v written to the paged bfloat16 cache.  Returns [T, (Hq + 2 Hkv) * hd]."""
+    _need_gpu(partials, positions, inv_freq, cache, block_table, seq_of_token)
+    width = (n_q_heads + 2 * n_kv_heads) * head_dim
+    if partials.dim() != 3 or partials.dtype != torch.float32 or partials.shape[2] != width or not partials.is_contiguous():
+        raise KernelError(f"partial sums must be a contiguous float32 [P, T, {width}] tensor")
+    n_part, n_tokens, _ = partials.shape
+    if head_dim % 8 != 0 or cache.dtype != torch.bfloat16:
+        raise KernelError("the rotation from partial sums takes head sizes of a multiple of 8 and a bfloat16 cache")
+    _i32(positions, "positions")
+    _i32(seq_of_token, "seq_of_token")
+    _i32(block_table, "block_table")
+    if inv_freq is not None and (inv_freq.dtype != torch.float32 or inv_freq.numel() != head_dim // 2 or not inv_freq.is_contiguous()):
+        raise KernelError(f"the rotary table must be float32 [{head_dim // 2}]")
+    if cache.dim() != 4 or cache.shape[1] != 2 or cache.shape[2] != n_kv_heads or cache.shape[3] % head_dim != 0 or not cache.is_contiguous():
+        raise KernelError(f"cache {tuple(cache.shape)} does not fit {n_kv_heads} heads of size {head_dim}")
+    if positions.numel() != n_tokens or seq_of_token.numel() != n_tokens or block_table.dim() != 2:
+        raise KernelError("positions and seq_of_token must be [T], block_table [B, W]")
+    out = torch.empty((n_tokens, width), dtype=torch.bfloat16, device=partials.device)
+    lib = _build.load("rope_kv")
+    _check(
+        lib,
+        lib.cwm_rope_kv_write_partials(
+            _ptr(out), ctypes.c_long(width), _ptr(partials), ctypes.c_int(n_part), ctypes.c_long(n_tokens * width),
+            _ptr(positions), _ptr(seq_of_token), _ptr(inv_freq), _ptr(cache), _ptr(block_table),
+            ctypes.c_int(block_table.shape[1]), ctypes.c_int(cache.shape[3] // head_dim), ctypes.c_int(cache.shape[0]),
+            ctypes.c_int(n_tokens), ctypes.c_int(n_q_heads), ctypes.c_int(n_kv_heads), ctypes.c_int(head_dim), _stream(),
+        ),
+    )
+    return out
 
 
 def sum_partials(partials: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:

@@ -950,3 +950,39 @@ def test_products_of_17_to_128_rows_take_the_tiled_kernel():
         ops.gemm_bf16_tile(xo, odd)
     x16 = x[:16].contiguous()
     assert torch.equal(ops.linear(x16, w), ops.gemm_bf16_stream(x16, w))
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,page_size,dim,m", [(4, 2, 16, 8, 64, 40), (6, 1, 64, 16, 128, 70), (12, 2, 128, 64, 256, 33), (3, 3, 48, 8, 192, 100)])
+def test_rope_kv_write_from_partial_sums(n_q, n_kv, hd, page_size, dim, m):
+    """The q/k/v projection of 17 to 128 rows leaves partial sums; rotation and cache write take them
+    as they are and give the bits of adding them first."""
+    from cwm_amd import ops
+
+    n_out = (n_q + 2 * n_kv) * hd
+    x = rnd((m, dim), torch.bfloat16, 1).to(DEV)
+    w = rnd((n_out, dim), torch.bfloat16, 2, 0.1).to(DEV)
+    inv_freq = plain.rope_frequencies(hd, 10000.0).to(DEV)
+    g = torch.Generator().manual_seed(5)
+    positions = torch.randint(0, 64, (m,), generator=g).to(torch.int32).to(DEV)
+    seq = torch.arange(m, dtype=torch.int32).to(DEV)
+    width = 64 // page_size + 1
+    table = torch.randperm(m * width, generator=g).to(torch.int32).reshape(m, width).contiguous().to(DEV)
+    caches = [torch.zeros((m * width, 2, n_kv, page_size * hd), dtype=torch.bfloat16, device=DEV) for _ in range(3)]
+    parts = rnd((3, m, n_out), torch.float32, 9, 1.5).to(DEV)
+    fused = ops.rope_kv_write_partials(parts, n_q, n_kv, hd, positions, inv_freq, caches[0], table, seq)
+    qkv = ops.sum_partials(parts, torch.bfloat16)
+    q = qkv[:, : n_q * hd].unflatten(1, (n_q, hd))
+    k = qkv[:, n_q * hd : (n_q + n_kv) * hd].unflatten(1, (n_kv, hd))
+    v = qkv[:, (n_q + n_kv) * hd :].unflatten(1, (n_kv, hd))
+    ops.rope_kv_write(q, k, v, positions, inv_freq, caches[1], table, seq)
+    assert torch.equal(fused, qkv)
+    assert torch.equal(caches[0], caches[1]) and caches[0].abs().sum() > 0
+    # and through the entry that the attention part calls, whatever the product leaves for these sizes
+    whole = ops.qkv_rope_write(x, w, None, n_q, n_kv, hd, positions, inv_freq, caches[2], table, seq)
+    plain_qkv = ops.linear(x, w)
+    q = plain_qkv[:, : n_q * hd].unflatten(1, (n_q, hd))
+    k = plain_qkv[:, n_q * hd : (n_q + n_kv) * hd].unflatten(1, (n_kv, hd))
+    v = plain_qkv[:, (n_q + n_kv) * hd :].unflatten(1, (n_kv, hd))
+    ops.rope_kv_write(q, k, v, positions, inv_freq, caches[1], table, seq)
+    assert torch.equal(whole, plain_qkv)
+    assert torch.equal(caches[2], caches[1])

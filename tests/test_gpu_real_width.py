@@ -68,7 +68,9 @@ def test_two_layers_of_the_32b_width(dtype):
         if k == 5:
             runner.admit("short")
         if k >= 5 and short_cur < len(short_toks):
-            m = min(130, len(short_toks) - short_cur)  # its prompt in portions beside the long request's decoded tokens
+            # its prompt in portions beside the long request's decoded tokens: steps of 131, 101 and 71 rows, which
+            # the products take in blocks of 128 rows twice, once, and in a block of 64
+            m = min([130, 100, 70][min(k - 5, 2)], len(short_toks) - short_cur)
             assert manager.extend("short", m)
             swant = sorted({0, m // 2, m - 1})
             portions.append(Portion("short", short_toks[short_cur : short_cur + m], swant))
