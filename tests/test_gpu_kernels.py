@@ -986,3 +986,32 @@ def test_rope_kv_write_from_partial_sums(n_q, n_kv, hd, page_size, dim, m):
     ops.rope_kv_write(q, k, v, positions, inv_freq, caches[1], table, seq)
     assert torch.equal(whole, plain_qkv)
     assert torch.equal(caches[2], caches[1])
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_gemm_bf16_tile_random_sizes(seed):
+    """Random row counts, widths, lengths of K and numbers of blocks: every cut of the work (tiles of
+    uneven width, tiles shared by many blocks or by none, blocks that run out of work) gives the product."""
+    import random
+
+    from cwm_amd import ops
+
+    rng = random.Random(seed)
+    for case in range(8):
+        m = rng.choice([1, 16, 17, 63, 64, 65, 127, 128, 129, 255, 300, 512])
+        n = 16 * rng.choice([1, 2, 5, 8, 9, 13, 24, 25, 77, 150, 333])
+        k = 64 * rng.choice([1, 2, 3, 7, 16, 33])
+        units = rng.choice([1, 2, 3, 5, 8, 13, 64, 256, 304])
+        a = rnd((m, k), torch.bfloat16, 100 * seed + case)
+        w = rnd((n, k), torch.bfloat16, 100 * seed + case + 50, 0.05)
+        want = a.double() @ w.double().T
+        limit = 1e-5 * float(want.abs().max()) * (1 + k / 512)
+        junk = torch.full((40, m, n), float("nan"), dtype=torch.float32, device=DEV)
+        del junk
+        parts = ops.gemm_bf16_tile(a.to(DEV), w.to(DEV), None, torch.float32, partials_ok=True, units=units).cpu()
+        total = parts.double().sum(0) if parts.dim() == 3 else parts.double()
+        assert (total - want).abs().max() <= limit, (m, n, k, units, tuple(parts.shape))
+        if n % 32 == 0:  # gate and up in groups of 8
+            got = ops.gemm_bf16_tile(a.to(DEV), w.to(DEV), None, torch.bfloat16, glu=True, units=units)
+            two = ops.silu_mul(ops.gemm_bf16_tile(a.to(DEV), w.to(DEV), None, torch.bfloat16, units=units), grouped=True)
+            assert torch.equal(got, two), (m, n, k, units)
