@@ -12,8 +12,8 @@
 // One block of four wavefronts per (token, key/value head, up to 8 of its query heads,
 // segment of the keys): a key and a value are loaded once and used for all the block's
 // query heads.  A token's keys are cut into segments by a rule of their number alone
-// (one segment up to 2,048 keys, then ceil(n / 2,048) segments, at most 16, of equal
-// length in chunks of 64); the wavefronts of a block take the segment's chunks of 64
+// (one segment up to 2,048 keys, then ceil(n / 1,024) segments, at most 16, of equal
+// length in chunks of 64: a window of 8,191 keys is read by eight blocks); the wavefronts of a block take the segment's chunks of 64
 // keys in turn (scores and softmax: a lane per key; values: a lane per dimension) and join
 // their results at the end in the order of the wavefronts; the segments of a token leave partial results (maximum, sum,
 // unnormalised output) that a second kernel joins in the order of the segments.
@@ -29,6 +29,7 @@ CWM_DEFINE_ERROR_API
 #define SIMPLE_WAVES 4      // wavefronts of a block: they take the segment's chunks of keys in turn
 #define SIMPLE_HEADS 8      // query heads of one key/value head that a block serves at once
 #define SIMPLE_SEGMENT 2048 // keys up to which a token has one segment
+#define SIMPLE_SEGMENT_LONG 1024 // keys of a segment, about, of a token with more (until there are SIMPLE_MAX_SEGMENTS)
 #define SIMPLE_MAX_SEGMENTS 16
 #define SIMPLE_D_REGS (SIMPLE_MAX_HEAD_DIM / CWM_WAVE)
 
@@ -44,7 +45,7 @@ __device__ __forceinline__ void wave_sync() {
 // segments of a token that reads n_keys keys, and their length (a multiple of 64)
 __device__ __forceinline__ int segments_of(int n_keys, int& seg_len) {
   int n_seg = 1;
-  if (n_keys > SIMPLE_SEGMENT) n_seg = min(SIMPLE_MAX_SEGMENTS, (n_keys + SIMPLE_SEGMENT - 1) / SIMPLE_SEGMENT);
+  if (n_keys > SIMPLE_SEGMENT) n_seg = min(SIMPLE_MAX_SEGMENTS, (n_keys + SIMPLE_SEGMENT_LONG - 1) / SIMPLE_SEGMENT_LONG);
   seg_len = ((n_keys + n_seg - 1) / n_seg + CWM_WAVE - 1) / CWM_WAVE * CWM_WAVE;
   return n_seg;
 }
@@ -373,7 +374,7 @@ extern "C" int cwm_attention_simple(const void* q, long q_stride, void* out, lon
   CWM_REQUIRE(max_keys >= 1, "attention: max_keys must be at least 1");
   if (n_tokens == 0) return 0;
   int max_segments = 1;
-  if (max_keys > SIMPLE_SEGMENT) max_segments = (max_keys + SIMPLE_SEGMENT - 1) / SIMPLE_SEGMENT;
+  if (max_keys > SIMPLE_SEGMENT) max_segments = (max_keys + SIMPLE_SEGMENT_LONG - 1) / SIMPLE_SEGMENT_LONG;  // as segments_of
   if (max_segments > SIMPLE_MAX_SEGMENTS) max_segments = SIMPLE_MAX_SEGMENTS;
   CWM_REQUIRE(max_segments == 1 || partial != nullptr, "attention: more than %d keys need the scratch for partial results",
               SIMPLE_SEGMENT);
