@@ -59,7 +59,8 @@ __global__ void rope_kv_write_bf16x8_kernel(bf16_t* __restrict__ q, long q_strid
       s[e] = 0.f;
       if (inv_freq) sincosf((float)pos * inv_freq[4 * piece + e], &s[e], &c[e]);
     }
-    for (int hh = threadIdx.y; hh < n_heads; hh += blockDim.y) {
+    // the blocks of a token (gridDim.y of them) take the heads in turn
+    for (int hh = blockIdx.y * blockDim.y + threadIdx.y; hh < n_heads; hh += gridDim.y * blockDim.y) {
       const bool is_key = hh >= n_q_heads;
       const int head = is_key ? hh - n_q_heads : hh;
       bf16_t* row = (is_key ? k + (size_t)t * k_stride : q + (size_t)t * q_stride) + (size_t)head * head_dim + 8 * piece;
@@ -92,8 +93,8 @@ __global__ void rope_kv_write_bf16x8_kernel(bf16_t* __restrict__ q, long q_strid
   }
   if ((vdst || PARTIALS) && v) {
     const int v_block = (page_size % 8 == 0) ? 8 : page_size;
-    const int tid = threadIdx.y * blockDim.x + threadIdx.x;
-    const int nthreads = blockDim.x * blockDim.y;
+    const int tid = (blockIdx.y * blockDim.y + threadIdx.y) * blockDim.x + threadIdx.x;
+    const int nthreads = gridDim.y * blockDim.x * blockDim.y;
     const int total = n_kv_heads * head_dim;
     bf16_t* vrow = v + (size_t)t * v_stride;
     for (int e = tid; e < total; e += nthreads) {
@@ -218,7 +219,9 @@ extern "C" int cwm_rope_kv_write(void* q, long q_stride, void* k, long k_stride,
     int py = 256 / px;
     if (py < 1) py = 1;
     if (py > heads) py = heads;
-    hipLaunchKernelGGL(rope_kv_write_bf16x8_kernel<false>, dim3(n_tokens), dim3(px, py), 0, stream, (bf16_t*)q, q_stride,
+    // few tokens: several blocks a token, so that a decode step's rows are not left to as many blocks
+    const int gy = n_tokens >= 1024 ? 1 : (heads + py - 1) / py;
+    hipLaunchKernelGGL(rope_kv_write_bf16x8_kernel<false>, dim3(n_tokens, gy), dim3(px, py), 0, stream, (bf16_t*)q, q_stride,
                        (bf16_t*)k, k_stride, (bf16_t*)v, v_stride, positions, seq_of_token, inv_freq, (bf16_t*)cache,
                        block_table, table_width, page_size, num_pages, n_q_heads, n_kv_heads, head_dim, (const float*)nullptr, 0,
                        0L);
@@ -266,7 +269,8 @@ extern "C" int cwm_rope_kv_write_partials(void* qkv, long qkv_stride, const floa
   bf16_t* q = (bf16_t*)qkv;
   bf16_t* k = q + (size_t)n_q_heads * head_dim;
   bf16_t* v = k + (size_t)n_kv_heads * head_dim;
-  hipLaunchKernelGGL(rope_kv_write_bf16x8_kernel<true>, dim3(n_tokens), dim3(px, py), 0, stream, q, qkv_stride, k, qkv_stride, v,
+  const int gy = n_tokens >= 1024 ? 1 : (n_q_heads + n_kv_heads + py - 1) / py;
+  hipLaunchKernelGGL(rope_kv_write_bf16x8_kernel<true>, dim3(n_tokens, gy), dim3(px, py), 0, stream, q, qkv_stride, k, qkv_stride, v,
                      qkv_stride, positions, seq_of_token, inv_freq, (bf16_t*)cache, block_table, table_width, page_size,
                      num_pages, n_q_heads, n_kv_heads, head_dim, partials, n_partials, partial_stride);
   return cwm_launch_status("rope_kv_write_partials");
