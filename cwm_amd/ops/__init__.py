@@ -193,10 +193,10 @@ def gate_up_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
     if fused:
         return gemm_bf16_stream(x, weight, bias, torch.bfloat16, glu=True)
     if (
-        grouped and x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+        grouped and bias is None and x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
         and STREAM_FUSED_ROWS < x.shape[0] <= TILE_ROWS and _tile_takes(x, weight)
     ):
-        return gemm_bf16_tile(x, weight, bias, torch.bfloat16, glu=True)
+        return gemm_bf16_tile(x, weight, None, torch.bfloat16, glu=True)
     return silu_mul(linear(x, weight, bias, partials_ok=True), out_dtype=x.dtype, grouped=grouped)
 
 
@@ -660,8 +660,8 @@ def gemm_bf16(
     m = x.shape[0]
     if not _stream_takes(x, weight):
         return gemm_f32(x, weight, bias, out_dtype)
-    if m > STREAM_FUSED_ROWS and _tile_wins(x, weight):
-        return gemm_bf16_tile(x, weight, bias, out_dtype, partials_ok)
+    if m > STREAM_FUSED_ROWS and bias is None and _tile_wins(x, weight):  # (the tiled kernel has no bias of its own)
+        return gemm_bf16_tile(x, weight, None, out_dtype, partials_ok)
     if m <= STREAM_MAX_ROWS:
         return gemm_bf16_stream(x, weight, bias, out_dtype, partials_ok)
     if out_dtype == torch.float32:
