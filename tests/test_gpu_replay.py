@@ -87,3 +87,27 @@ def test_first_tokens_and_long_decoding(folders, plain_cache, dtype):
     local = [g.index for g in rep.manager.groups if g.window is not None]
     for g in local:
         assert rep.manager.pages_held("x")[g] <= (8 - 1 + 1 + 3) // 4 + 1
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_many_requests_decode_together(folders, dtype):
+    """Ninety requests in one batch: their prompts in one step of 270 rows, five steps of 90 single
+    tokens, then, fifty of them ended, five steps of 40: the row counts at which the products change
+    kernels (blocks of 128 rows, of 64, the library above 256)."""
+    from cwm_amd.replay import Replayer
+
+    name = "tiny_a"
+    vocab = configs.get(name)["vocab_size"]
+    requests = {f"q{i}": traces.random_tokens(1000 + i, 3 + 5 + (5 if i < 40 else 0), vocab) for i in range(90)}
+    steps = [{"step": 0, "entries": [{"id": rid, "tokens": toks[:3], "want": [0, 1, 2]} for rid, toks in requests.items()], "end": []}]
+    for k in range(5):
+        steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": [toks[3 + k]], "want": [0]} for rid, toks in requests.items()],
+                      "end": [f"q{i}" for i in range(40, 90)] if k == 4 else []})
+    for k in range(5):
+        steps.append({"step": len(steps), "entries": [{"id": f"q{i}", "tokens": [requests[f"q{i}"][8 + k]], "want": [0]} for i in range(40)],
+                      "end": [f"q{i}" for i in range(40)] if k == 4 else []})
+    rep = Replayer(folders[name, dtype], dtype, 90 * 64, page_size=8, max_requests=90, poison_freed_pages=True)
+    outputs = traces.run_in_process(rep, steps)
+    got = traces.gather(steps, outputs, {k: len(v) for k, v in requests.items()}, vocab)
+    compare(got, cmp.expected(folders[name, dtype], requests, dtype), dtype, f"{name} {dtype} ninety requests")
+    assert rep.manager.live_requests() == []
