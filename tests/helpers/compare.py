@@ -12,7 +12,11 @@ distance from the exact logits is another draw of the same size: over 2,052
 requests of random configurations (1 to 24 layers, weights of std 0.02 to 0.1, every
 way of cutting the work) the ratio of the two root-mean-square errors had median
 1.00 and maximum 1.33, the ratio of the two largest errors median 1.00 and maximum
-2.12.  A request passes with ratios of at most 1.5 and 3.
+2.12.  A request passes with ratios of at most 1.5 and 3.  (A later search over 7,491
+requests, more of them with 16 and 24 layers, had the same medians, 99th percentiles
+of 1.14 and 1.34, and maxima of 1.52 and 1.89: the highest on requests of one or two
+tokens and a vocabulary of 97, where both errors are estimated from a few hundred
+logits.  The limits are as they were.)
 """
 
 from __future__ import annotations
