@@ -467,6 +467,9 @@ attention_lds_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __rest
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // the key/value head changes fastest with the block's number: workgroups go to the chip's eight XCDs in turn,
+  // so with eight (or four, two) key/value heads the blocks of one head run on the same XCD(s) and find the keys
+  // and values that the head's other blocks fetched in that XCD's L2
   const int item = blockIdx.x / n_kv_heads_grid;
   const int g = blockIdx.x - item * n_kv_heads_grid;
   const int* w = work + (size_t)item * WORK_INTS;
