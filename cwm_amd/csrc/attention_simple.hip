@@ -53,20 +53,22 @@ __device__ __forceinline__ int segments_of(int n_keys, int& seg_len) {
 // partial result of (token, query head, segment): [head_dim] unnormalised output, then maximum and sum
 #define PARTIAL_STRIDE(hd) ((hd) + 2)
 
-template <typename T>
+// HEADS: query heads a block serves (at most HEADS); D_REGS: dimensions of a head per lane (head sizes up to
+// 64 * D_REGS).  The arithmetic is the same for every pair; smaller ones leave registers for more wavefronts.
+template <typename T, int HEADS, int D_REGS>
 __global__ void __launch_bounds__(SIMPLE_WAVES * CWM_WAVE)
 attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out, long out_stride,
                         const T* __restrict__ cache, const int* __restrict__ block_table, int table_width,
                         const int* __restrict__ positions, const int* __restrict__ seq_of_token, float* __restrict__ partial,
                         int n_q_heads, int n_kv_heads, int head_groups, int head_dim, int page_size, int num_pages,
                         int window_left, float scale) {
-  __shared__ __attribute__((aligned(16))) float qs[SIMPLE_HEADS][SIMPLE_MAX_HEAD_DIM];
+  __shared__ __attribute__((aligned(16))) float qs[HEADS][D_REGS * CWM_WAVE];
   // probabilities of a chunk, key jj at [in0 + jj] (in0: the first key's place in its block of 8 values), so that the
   // eight of a block lie at a multiple of 8
-  __shared__ __attribute__((aligned(16))) float ps_all[SIMPLE_WAVES][SIMPLE_HEADS][CWM_WAVE + 8];
+  __shared__ __attribute__((aligned(16))) float ps_all[SIMPLE_WAVES][HEADS][CWM_WAVE + 8];
   __shared__ long long voff_all[SIMPLE_WAVES][CWM_WAVE];
-  __shared__ float part_m[SIMPLE_WAVES][SIMPLE_HEADS], part_l[SIMPLE_WAVES][SIMPLE_HEADS];
-  __shared__ float part_o[SIMPLE_WAVES][SIMPLE_HEADS][SIMPLE_MAX_HEAD_DIM];
+  __shared__ float part_m[SIMPLE_WAVES][HEADS], part_l[SIMPLE_WAVES][HEADS];
+  __shared__ float part_o[SIMPLE_WAVES][HEADS][D_REGS * CWM_WAVE];
 
   const int lane = threadIdx.x & (CWM_WAVE - 1);
   const int wave = threadIdx.x / CWM_WAVE;
@@ -103,14 +105,14 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
 
   float* ps = &ps_all[wave][0][0];
   long long* voff = voff_all[wave];
-  float m[SIMPLE_HEADS], l[SIMPLE_HEADS];
-  float o[SIMPLE_HEADS][SIMPLE_D_REGS];
+  float m[HEADS], l[HEADS];
+  float o[HEADS][D_REGS];
 #pragma unroll
-  for (int h = 0; h < SIMPLE_HEADS; ++h) {
+  for (int h = 0; h < HEADS; ++h) {
     m[h] = neg_inf;
     l[h] = 0.f;
 #pragma unroll
-    for (int r = 0; r < SIMPLE_D_REGS; ++r) o[h][r] = 0.f;
+    for (int r = 0; r < D_REGS; ++r) o[h][r] = 0.f;
   }
 
   // wavefront w takes the chunks of 64 keys w, w + SIMPLE_WAVES, ... of the segment
@@ -119,9 +121,9 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
     const bool valid = j < k1;
     const int n = min(CWM_WAVE, k1 - base);
     const int in0 = base & 7;  // the first key's place in its block of 8 values
-    float s[SIMPLE_HEADS];
+    float s[HEADS];
 #pragma unroll
-    for (int h = 0; h < SIMPLE_HEADS; ++h) s[h] = neg_inf;
+    for (int h = 0; h < HEADS; ++h) s[h] = neg_inf;
     long long vo = -1;
     if (valid) {
       const int lp = j / page_size;
@@ -129,12 +131,12 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
       const int page = lp < table_width ? block_table[(size_t)b * table_width + lp] : -1;
       if (page < 0 || page >= num_pages) {
 #pragma unroll
-        for (int h = 0; h < SIMPLE_HEADS; ++h) s[h] = nan;  // a key that should be there has no page: make it show
+        for (int h = 0; h < HEADS; ++h) s[h] = nan;  // a key that should be there has no page: make it show
       } else {
         const T* krow = cache + (size_t)page * 2 * plane + ((size_t)g * page_size + slot) * head_dim;
-        float dot[SIMPLE_HEADS];
+        float dot[HEADS];
 #pragma unroll
-        for (int h = 0; h < SIMPLE_HEADS; ++h) dot[h] = 0.f;
+        for (int h = 0; h < HEADS; ++h) dot[h] = 0.f;
         if (sizeof(T) == 4 && vec4) {
           // sixteen values per round of loads; every sum keeps the order d = 0, 1, 2, ...
           int d = 0;
@@ -145,7 +147,7 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
 #pragma unroll
-              for (int h = 0; h < SIMPLE_HEADS; ++h) {
+              for (int h = 0; h < HEADS; ++h) {
                 if (h < nh) {
                   const float4 qv = *(const float4*)(&qs[h][d + 4 * u]);
                   dot[h] = fmaf(qv.x, kv[u].x, dot[h]);
@@ -159,7 +161,7 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
           for (; d < head_dim; d += 4) {
             const float4 kv = *(const float4*)((const float*)krow + d);
 #pragma unroll
-            for (int h = 0; h < SIMPLE_HEADS; ++h) {
+            for (int h = 0; h < HEADS; ++h) {
               if (h < nh) {
                 const float4 qv = *(const float4*)(&qs[h][d]);
                 dot[h] = fmaf(qv.x, kv.x, dot[h]);
@@ -173,20 +175,20 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
           for (int d = 0; d < head_dim; ++d) {
             const float kd = Elem<T>::load(krow + d);
 #pragma unroll
-            for (int h = 0; h < SIMPLE_HEADS; ++h)
+            for (int h = 0; h < HEADS; ++h)
               if (h < nh) dot[h] = fmaf(qs[h][d], kd, dot[h]);
           }
         }
 #pragma unroll
-        for (int h = 0; h < SIMPLE_HEADS; ++h) s[h] = dot[h] * scale;
+        for (int h = 0; h < HEADS; ++h) s[h] = dot[h] * scale;
         // values: blocks of v_block keys, [slot / v_block][dim][slot % v_block]
         vo = (long long)((size_t)page * 2 * plane + plane + (size_t)g * head_dim * page_size +
                          (size_t)(slot / v_block) * head_dim * v_block + slot % v_block);
       }
     }
-    float alpha[SIMPLE_HEADS];
+    float alpha[HEADS];
 #pragma unroll
-    for (int h = 0; h < SIMPLE_HEADS; ++h) {
+    for (int h = 0; h < HEADS; ++h) {
       if (h < nh) {
         const float mx = wave_max(s[h]);
         const float m_new = fmaxf(m[h], mx);
@@ -202,12 +204,12 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
     voff[lane] = vo;
     wave_sync();  // the wavefront's own lanes read these next
 #pragma unroll
-    for (int r = 0; r < SIMPLE_D_REGS; ++r) {
+    for (int r = 0; r < D_REGS; ++r) {
       const int d = lane + r * CWM_WAVE;
       if (d < head_dim) {
-        float acc[SIMPLE_HEADS];
+        float acc[HEADS];
 #pragma unroll
-        for (int h = 0; h < SIMPLE_HEADS; ++h) acc[h] = o[h][r] * alpha[h];
+        for (int h = 0; h < HEADS; ++h) acc[h] = o[h][r] * alpha[h];
         if (sizeof(T) == 4 && vec4 && v_block == 8) {
           // the eight keys of a block of values lie side by side for one dimension: two loads serve up to
           // eight keys.  The chunk's 64 keys lie in at most nine such blocks; all their loads are issued
@@ -230,9 +232,9 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
           for (int blk = 0; blk < 9; ++blk) {
             if (8 * blk - in0 >= n) break;
             const float vv[8] = {lo[blk].x, lo[blk].y, lo[blk].z, lo[blk].w, hi[blk].x, hi[blk].y, hi[blk].z, hi[blk].w};
-            float pp[SIMPLE_HEADS][8];
+            float pp[HEADS][8];
 #pragma unroll
-            for (int h = 0; h < SIMPLE_HEADS; ++h) {
+            for (int h = 0; h < HEADS; ++h) {
               if (h < nh) {
                 const float4 pl = *(const float4*)(&ps[h * (CWM_WAVE + 8) + 8 * blk]);
                 const float4 ph = *(const float4*)(&ps[h * (CWM_WAVE + 8) + 8 * blk + 4]);
@@ -245,7 +247,7 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
               const int jj = 8 * blk + x - in0;
               if (jj >= 0 && jj < n) {
 #pragma unroll
-                for (int h = 0; h < SIMPLE_HEADS; ++h)
+                for (int h = 0; h < HEADS; ++h)
                   if (h < nh) acc[h] = fmaf(pp[h][x], vv[x], acc[h]);
               }
             }
@@ -255,12 +257,12 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
             const long long off = voff[jj];
             const float vv = off >= 0 ? Elem<T>::load(cache + off + (size_t)d * v_block) : nan;
 #pragma unroll
-            for (int h = 0; h < SIMPLE_HEADS; ++h)
+            for (int h = 0; h < HEADS; ++h)
               if (h < nh) acc[h] = fmaf(ps[h * (CWM_WAVE + 8) + in0 + jj], vv, acc[h]);
           }
         }
 #pragma unroll
-        for (int h = 0; h < SIMPLE_HEADS; ++h) o[h][r] = acc[h];
+        for (int h = 0; h < HEADS; ++h) o[h][r] = acc[h];
       }
     }
     wave_sync();
@@ -268,14 +270,14 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
 
   // the wavefronts' results, joined in the order of the wavefronts
 #pragma unroll
-  for (int h = 0; h < SIMPLE_HEADS; ++h) {
+  for (int h = 0; h < HEADS; ++h) {
     if (h < nh) {
       if (lane == 0) {
         part_m[wave][h] = m[h];
         part_l[wave][h] = l[h];
       }
 #pragma unroll
-      for (int r = 0; r < SIMPLE_D_REGS; ++r) {
+      for (int r = 0; r < D_REGS; ++r) {
         const int d = lane + r * CWM_WAVE;
         if (d < head_dim) part_o[wave][h][d] = o[h][r];
       }
@@ -297,7 +299,7 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
     T* orow = out + (size_t)t * out_stride + (size_t)(h0 + h) * head_dim;
     float* prow = n_seg > 1 ? partial + (((size_t)t * n_q_heads + h0 + h) * SIMPLE_MAX_SEGMENTS + seg) * PARTIAL_STRIDE(head_dim) : nullptr;
 #pragma unroll
-    for (int r = 0; r < SIMPLE_D_REGS; ++r) {
+    for (int r = 0; r < D_REGS; ++r) {
       const int d = lane + r * CWM_WAVE;
       if (d < head_dim) {
         float sum = 0.f;
@@ -386,15 +388,37 @@ extern "C" int cwm_attention_simple(const void* q, long q_stride, void* out, lon
   CWM_REQUIRE(join_blocks <= 0x7fffffffLL, "attention: too many (token, head) pairs: %lld", join_blocks);
   dim3 grid((unsigned)blocks, (unsigned)max_segments);
   if (dtype == CWM_F32) {
-    hipLaunchKernelGGL(attention_simple_kernel<float>, grid, dim3(SIMPLE_WAVES * CWM_WAVE), 0, stream, (const float*)q,
-                       q_stride, (float*)out, out_stride, (const float*)cache, block_table, table_width, positions,
-                       seq_of_token, partial, n_q_heads, n_kv_heads, head_groups, head_dim, page_size, num_pages, window_left,
-                       scale);
+    // the smallest block shape that holds the heads of a group and the head size
+    const int heads = group < SIMPLE_HEADS ? group : SIMPLE_HEADS;
+#define CWM_LAUNCH_SIMPLE(HEADS, D_REGS)                                                                                   \
+  hipLaunchKernelGGL((attention_simple_kernel<float, HEADS, D_REGS>), grid, dim3(SIMPLE_WAVES * CWM_WAVE), 0, stream,     \
+                     (const float*)q, q_stride, (float*)out, out_stride, (const float*)cache, block_table, table_width,   \
+                     positions, seq_of_token, partial, n_q_heads, n_kv_heads, head_groups, head_dim, page_size, num_pages, \
+                     window_left, scale)
+#define CWM_LAUNCH_SIMPLE_HEADS(D_REGS)   \
+  do {                                    \
+    if (heads <= 2)                       \
+      CWM_LAUNCH_SIMPLE(2, D_REGS);       \
+    else if (heads <= 4)                  \
+      CWM_LAUNCH_SIMPLE(4, D_REGS);       \
+    else if (heads <= 6)                  \
+      CWM_LAUNCH_SIMPLE(6, D_REGS);       \
+    else                                  \
+      CWM_LAUNCH_SIMPLE(SIMPLE_HEADS, D_REGS); \
+  } while (0)
+    if (head_dim <= CWM_WAVE)
+      CWM_LAUNCH_SIMPLE_HEADS(1);
+    else if (head_dim <= 2 * CWM_WAVE)
+      CWM_LAUNCH_SIMPLE_HEADS(2);
+    else
+      CWM_LAUNCH_SIMPLE_HEADS(SIMPLE_D_REGS);
+#undef CWM_LAUNCH_SIMPLE_HEADS
+#undef CWM_LAUNCH_SIMPLE
     if (max_segments > 1)
       hipLaunchKernelGGL(attention_simple_join_kernel<float>, dim3((unsigned)join_blocks), dim3(CWM_WAVE), 0, stream,
                          (float*)out, out_stride, (const float*)partial, positions, n_q_heads, head_dim, window_left);
   } else if (dtype == CWM_BF16) {
-    hipLaunchKernelGGL(attention_simple_kernel<bf16_t>, grid, dim3(SIMPLE_WAVES * CWM_WAVE), 0, stream, (const bf16_t*)q,
+    hipLaunchKernelGGL((attention_simple_kernel<bf16_t, SIMPLE_HEADS, SIMPLE_D_REGS>), grid, dim3(SIMPLE_WAVES * CWM_WAVE), 0, stream, (const bf16_t*)q,
                        q_stride, (bf16_t*)out, out_stride, (const bf16_t*)cache, block_table, table_width, positions,
                        seq_of_token, partial, n_q_heads, n_kv_heads, head_groups, head_dim, page_size, num_pages, window_left,
                        scale);
