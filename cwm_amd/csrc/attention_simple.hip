@@ -31,6 +31,9 @@ CWM_DEFINE_ERROR_API
 #define SIMPLE_SEGMENT 2048 // keys up to which a token has one segment
 #define SIMPLE_SEGMENT_LONG 1024 // keys of a segment, about, of a token with more (until there are SIMPLE_MAX_SEGMENTS)
 #define SIMPLE_MAX_SEGMENTS 16
+#ifndef SIMPLE_V_ROUND
+#define SIMPLE_V_ROUND 5     // blocks of 8 values whose loads are in flight together
+#endif
 #define SIMPLE_D_REGS (SIMPLE_MAX_HEAD_DIM / CWM_WAVE)
 
 extern "C" int cwm_attention_simple_max_segments() { return SIMPLE_MAX_SEGMENTS; }
@@ -212,43 +215,49 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
         for (int h = 0; h < HEADS; ++h) acc[h] = o[h][r] * alpha[h];
         if (sizeof(T) == 4 && vec4 && v_block == 8) {
           // the eight keys of a block of values lie side by side for one dimension: two loads serve up to
-          // eight keys.  The chunk's 64 keys lie in at most nine such blocks; all their loads are issued
+          // eight keys.  The chunk's 64 keys lie in at most nine such blocks; the loads of several are issued
           // before the first is used; every sum keeps the order of the keys.
-          float4 lo[9], hi[9];
+          // (SIMPLE_V_ROUND blocks a round of loads: the registers that nine would take cost a wavefront per SIMD)
 #pragma unroll
-          for (int blk = 0; blk < 9; ++blk) {
-            const int jj = max(0, 8 * blk - in0);  // the block's first key of this chunk
-            lo[blk] = hi[blk] = make_float4(nan, nan, nan, nan);
-            if (jj < n && (blk < 8 || in0 > 0)) {
-              const long long off = voff[jj];
-              if (off >= 0) {
-                const float* vb = (const float*)cache + (off - ((base + jj) & 7)) + (size_t)d * 8;
-                lo[blk] = *(const float4*)vb;
-                hi[blk] = *(const float4*)(vb + 4);
-              }
-            }
-          }
+          for (int b0 = 0; b0 < 9; b0 += SIMPLE_V_ROUND) {
+            float4 lo[SIMPLE_V_ROUND], hi[SIMPLE_V_ROUND];
 #pragma unroll
-          for (int blk = 0; blk < 9; ++blk) {
-            if (8 * blk - in0 >= n) break;
-            const float vv[8] = {lo[blk].x, lo[blk].y, lo[blk].z, lo[blk].w, hi[blk].x, hi[blk].y, hi[blk].z, hi[blk].w};
-            float pp[HEADS][8];
-#pragma unroll
-            for (int h = 0; h < HEADS; ++h) {
-              if (h < nh) {
-                const float4 pl = *(const float4*)(&ps[h * (CWM_WAVE + 8) + 8 * blk]);
-                const float4 ph = *(const float4*)(&ps[h * (CWM_WAVE + 8) + 8 * blk + 4]);
-                pp[h][0] = pl.x; pp[h][1] = pl.y; pp[h][2] = pl.z; pp[h][3] = pl.w;
-                pp[h][4] = ph.x; pp[h][5] = ph.y; pp[h][6] = ph.z; pp[h][7] = ph.w;
+            for (int u = 0; u < SIMPLE_V_ROUND; ++u) {
+              const int blk = b0 + u;
+              const int jj = max(0, 8 * blk - in0);  // the block's first key of this chunk
+              lo[u] = hi[u] = make_float4(nan, nan, nan, nan);
+              if (blk < 9 && jj < n && (blk < 8 || in0 > 0)) {
+                const long long off = voff[jj];
+                if (off >= 0) {
+                  const float* vb = (const float*)cache + (off - ((base + jj) & 7)) + (size_t)d * 8;
+                  lo[u] = *(const float4*)vb;
+                  hi[u] = *(const float4*)(vb + 4);
+                }
               }
             }
 #pragma unroll
-            for (int x = 0; x < 8; ++x) {
-              const int jj = 8 * blk + x - in0;
-              if (jj >= 0 && jj < n) {
+            for (int u = 0; u < SIMPLE_V_ROUND; ++u) {
+              const int blk = b0 + u;
+              if (blk >= 9 || 8 * blk - in0 >= n) break;
+              const float vv[8] = {lo[u].x, lo[u].y, lo[u].z, lo[u].w, hi[u].x, hi[u].y, hi[u].z, hi[u].w};
+              float pp[HEADS][8];
 #pragma unroll
-                for (int h = 0; h < HEADS; ++h)
-                  if (h < nh) acc[h] = fmaf(pp[h][x], vv[x], acc[h]);
+              for (int h = 0; h < HEADS; ++h) {
+                if (h < nh) {
+                  const float4 pl = *(const float4*)(&ps[h * (CWM_WAVE + 8) + 8 * blk]);
+                  const float4 ph = *(const float4*)(&ps[h * (CWM_WAVE + 8) + 8 * blk + 4]);
+                  pp[h][0] = pl.x; pp[h][1] = pl.y; pp[h][2] = pl.z; pp[h][3] = pl.w;
+                  pp[h][4] = ph.x; pp[h][5] = ph.y; pp[h][6] = ph.z; pp[h][7] = ph.w;
+                }
+              }
+#pragma unroll
+              for (int x = 0; x < 8; ++x) {
+                const int jj = 8 * blk + x - in0;
+                if (jj >= 0 && jj < n) {
+#pragma unroll
+                  for (int h = 0; h < HEADS; ++h)
+                    if (h < nh) acc[h] = fmaf(pp[h][x], vv[x], acc[h]);
+                }
               }
             }
           }
