@@ -31,6 +31,9 @@ CWM_DEFINE_ERROR_API
 #define SIMPLE_SEGMENT 2048 // keys up to which a token has one segment
 #define SIMPLE_SEGMENT_LONG 1024 // keys of a segment, about, of a token with more (until there are SIMPLE_MAX_SEGMENTS)
 #define SIMPLE_MAX_SEGMENTS 16
+#ifndef SIMPLE_K_ROUND
+#define SIMPLE_K_ROUND 8     // 16-byte loads of a key's row that are in flight together
+#endif
 #ifndef SIMPLE_V_ROUND
 #define SIMPLE_V_ROUND 5     // blocks of 8 values whose loads are in flight together
 #endif
@@ -141,14 +144,14 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
 #pragma unroll
         for (int h = 0; h < HEADS; ++h) dot[h] = 0.f;
         if (sizeof(T) == 4 && vec4) {
-          // sixteen values per round of loads; every sum keeps the order d = 0, 1, 2, ...
+          // 4 * SIMPLE_K_ROUND values per round of loads; every sum keeps the order d = 0, 1, 2, ...
           int d = 0;
-          for (; d + 16 <= head_dim; d += 16) {
-            float4 kv[4];
+          for (; d + 4 * SIMPLE_K_ROUND <= head_dim; d += 4 * SIMPLE_K_ROUND) {
+            float4 kv[SIMPLE_K_ROUND];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) kv[u] = *(const float4*)((const float*)krow + d + 4 * u);
+            for (int u = 0; u < SIMPLE_K_ROUND; ++u) kv[u] = *(const float4*)((const float*)krow + d + 4 * u);
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < SIMPLE_K_ROUND; ++u) {
 #pragma unroll
               for (int h = 0; h < HEADS; ++h) {
                 if (h < nh) {
