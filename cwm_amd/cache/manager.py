@@ -20,7 +20,7 @@ still reads window-1 keys before it.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, Hashable, List, Mapping, Optional, Sequence, Tuple, Union
+from typing import Dict, Hashable, List, Mapping, Optional, Sequence, Union
 
 from ..parts.base import CacheSpec, PagedKVSpec, StateSpec
 from .pages import GroupTable, OutOfPages, PageAccountingError, PagePool, pages_for

@@ -11,7 +11,7 @@ window of keys gives a page back as soon as no later query can reach it.
 from __future__ import annotations
 
 import heapq
-from typing import Dict, List, Optional
+from typing import List, Optional
 
 
 class OutOfPages(RuntimeError):

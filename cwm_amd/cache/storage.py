@@ -12,7 +12,7 @@ of one row-major tensor per layer (cwm/fastgen/utils/cache.py:85-97,131-132).
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, List, Optional, Sequence
+from typing import Dict, Optional, Sequence
 
 import torch
 

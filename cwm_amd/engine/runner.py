@@ -17,7 +17,7 @@ import torch
 from ..cache.manager import CacheManager
 from ..cache.storage import CacheStorage
 from ..models.model import Model
-from .batch import BatchError, Portion, StepBatch, build_batch
+from .batch import Portion, build_batch
 
 
 class ModelRunner:

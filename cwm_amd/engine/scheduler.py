@@ -31,10 +31,9 @@ from __future__ import annotations
 
 from collections import deque
 from dataclasses import dataclass, field
-from typing import Any, Callable, Deque, Dict, Hashable, List, Optional, Sequence, Set
+from typing import Any, Callable, Deque, Hashable, List, Optional, Sequence, Set
 
 from ..cache.manager import CacheManager
-from ..cache.pages import pages_for
 from .batch import Portion
 
 WAITING, RUNNING, PARKED, FINISHED = "waiting", "running", "parked", "finished"

@@ -11,7 +11,7 @@ batch, and a preempted request goes on with its stream where it was.
 from __future__ import annotations
 
 import hashlib
-from typing import Any, Hashable, List, Optional, Sequence, Tuple
+from typing import Any, List, Sequence, Tuple
 
 import numpy as np
 import torch
