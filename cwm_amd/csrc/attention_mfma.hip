@@ -443,11 +443,6 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __res
 #define DMA_TILE_BYTES (2 * DMA_K_BYTES)
 #define DMA_HEAD_DIM_OK (HEAD_DIM == 64 || HEAD_DIM == 128)
 
-// every lane's 16 bytes at base + offset go to LDS byte address lds + 16 * lane (lds is uniform)
-__device__ __forceinline__ void dma16(const bf16_t* base, uint32_t offset, uint32_t lds) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(offset), "s"(base) : "memory", "m0");
-}
-
 // MIN_BLOCKS blocks share a compute unit.  With two (at most 256 registers a wavefront) or three
 // (168) the compiler keeps the matrix-core accumulators in ordinary vector registers; from the
 // accumulation registers every rescaling would cost a copy out and a copy back.

@@ -88,6 +88,14 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
   return total;
 }
 
+// Direct load from global memory into LDS (global_load_lds_dwordx4): every lane's 16 bytes at
+// base + offset go to LDS byte address lds + 16 * lane (base and lds are uniform over the
+// wavefront).  The load counts in vmcnt like any other; the compiler does not know of it, so
+// whoever issues it also writes the waits (s_waitcnt vmcnt) before the LDS is read.
+__device__ __forceinline__ void dma16(const bf16_t* base, uint32_t offset, uint32_t lds) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(offset), "s"(base) : "memory", "m0");
+}
+
 // ---- host side: error channel ------------------------------------------------ //
 static thread_local char cwm_error_buffer[512] = {0};
 

@@ -55,11 +55,6 @@ union Frag8 {
 
 extern "C" int cwm_gemm_bf16_tile_max_rows() { return TL_MAX_ROWS; }
 
-// every lane's 16 bytes at base + offset go to LDS byte address lds + 16 * lane (lds is uniform)
-__device__ __forceinline__ void dma16(const bf16_t* base, uint32_t offset, uint32_t lds) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(offset), "s"(base) : "memory", "m0");
-}
-
 #ifndef TL_WAVES_64
 #define TL_WAVES_64 8  // wavefronts of a block of 64 rows
 #endif
