@@ -52,15 +52,6 @@ CWM_DEFINE_ERROR_API
 #define WORK_INTS 6
 #define PARTIAL_STRIDE (HEAD_DIM + 4)  // max and sum after the output; keeps rows 16-byte aligned
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float float4v __attribute__((ext_vector_type(4)));
-
-union Frag8 {
-  uint4 u;
-  bf16x8 v;
-  uint16_t h[8];
-};
-
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) { return pack2_bf16(lo, hi); }
 
 // One row's share of a 32-key tile of scores: masks (only where a tile reaches past some

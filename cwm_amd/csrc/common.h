@@ -88,6 +88,17 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
   return total;
 }
 
+// Operands and results of the matrix-core instructions: eight bfloat16 values of one lane
+// (16 bytes, also as one load) and the four float32 sums of one lane.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+union Frag8 {
+  uint4 u;
+  bf16x8 v;
+  uint16_t h[8];
+};
+
 // Direct load from global memory into LDS (global_load_lds_dwordx4): every lane's 16 bytes at
 // base + offset go to LDS byte address lds + 16 * lane (base and lds are uniform over the
 // wavefront).  The load counts in vmcnt like any other; the compiler does not know of it, so

@@ -29,14 +29,6 @@
 
 CWM_DEFINE_ERROR_API
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float float4v __attribute__((ext_vector_type(4)));
-
-union Frag8 {
-  uint4 u;
-  bf16x8 v;
-};
-
 // block shapes: {tiles of A, wavefronts, steps of 32 along K in half a W tile}; a wavefront
 // holds 2 * half steps of each of its tiles of A in registers
 #ifndef ST1_WAVES

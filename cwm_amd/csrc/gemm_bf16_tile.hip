@@ -37,14 +37,6 @@
 
 CWM_DEFINE_ERROR_API
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float float4v __attribute__((ext_vector_type(4)));
-
-union Frag8 {
-  uint4 u;
-  bf16x8 v;
-};
-
 #define TL_GROUPS 12        // groups of 16 columns in the widest tile
 #ifndef TL_SHARED_GROUPS
 #define TL_SHARED_GROUPS 8  // in a tile whose steps several blocks share

@@ -26,8 +26,6 @@
 
 CWM_DEFINE_ERROR_API
 
-typedef float float4v __attribute__((ext_vector_type(4)));
-
 #define FS_WAVES 16
 #define FS_HALF 6  // steps of 16 along K in half a tile of W; a wavefront holds 2 * FS_HALF steps of A
 
