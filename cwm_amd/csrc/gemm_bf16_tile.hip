@@ -113,10 +113,16 @@ gemm_tile_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restric
     asrc = A + (size_t)m0 * lda;
   };
   enter_tile(i_tile);
+  // Blocks that own whole tiles all start at a tile's first step: they would ask the L2 for the same lines of A at
+  // the same time.  Each walks K from a start of its own instead (and round to it); a sum's order is then fixed by
+  // the block's number, that is by the column, as before by the cut.
+  const int rotation = __builtin_amdgcn_readfirstlane(slabs == 1 ? (int)((blockIdx.x * 37u) % (unsigned)steps) : 0);
   const uint32_t lds0 = (uint32_t)(uintptr_t)(&lds[0]);
   auto issue = [&](int buf) {
-    const bf16_t* ws = wsrc + (size_t)i_step * TL_BK;
-    const bf16_t* as = asrc + (size_t)i_step * TL_BK;
+    int k_step = i_step + rotation;  // where along K this step reads
+    if (k_step >= steps) k_step -= steps;
+    const bf16_t* ws = wsrc + (size_t)k_step * TL_BK;
+    const bf16_t* as = asrc + (size_t)k_step * TL_BK;
     const uint32_t dst = lds0 + buf * STAGE;
 #pragma unroll
     for (int i = 0; i < W_DMA; ++i) dma16(ws, w_off[i], dst + (wave * W_DMA + i) * 1024);
