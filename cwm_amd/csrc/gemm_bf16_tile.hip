@@ -43,6 +43,7 @@ CWM_DEFINE_ERROR_API
 #endif
 #define TL_MIN_GROUPS 6     // narrower whole tiles would load more of A than of W
 #define TL_BK 64
+#define TL_ROTATE_STEPS 128   // steps of K up to which the tiles walk K from different starts
 #define TL_MAX_ROWS 512
 
 extern "C" int cwm_gemm_bf16_tile_max_rows() { return TL_MAX_ROWS; }
@@ -91,6 +92,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restric
   const bf16_t* wsrc;
   const bf16_t* asrc;
   uint32_t w_off[W_DMA], a_off[A_DMA];
+  int rotation = 0;
   // this lane's pieces of a step: load q fills rows 8 q .. 8 q + 7; rows past the tile or the matrix read its last row
   auto enter_tile = [&](int tile) {
     const int ct = tile / n_row_blocks;
@@ -111,15 +113,18 @@ gemm_tile_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restric
     }
     wsrc = W + (size_t)n0 * ldw;
     asrc = A + (size_t)m0 * lda;
+    // Blocks that are at the same step of their tiles ask the L2 for the same lines of A at the same time (blocks
+    // that own whole tiles all start at step 0).  With a short K, where A stays in the L2, that costs more than it
+    // saves (gate/up of the 32B shape at 64 rows: 106 against 96 us; an 8,192 x 8,192 product 38 against 28), so a
+    // tile's step j reads K at (j + rotation) mod steps, with a rotation of the tile's own.  With a long K the W that
+    // streams through the L2 pushes A out between its uses, and blocks in step fetch a line once for all of them
+    // (down, K = 21,504: 51 against 54 us), so there is no rotation.  A sum's order is fixed by its tile and the cut.
+    rotation = steps <= TL_ROTATE_STEPS ? __builtin_amdgcn_readfirstlane((int)(((unsigned)tile * 37u) % (unsigned)steps)) : 0;
   };
   enter_tile(i_tile);
-  // Blocks that own whole tiles all start at a tile's first step: they would ask the L2 for the same lines of A at
-  // the same time.  Each walks K from a start of its own instead (and round to it); a sum's order is then fixed by
-  // the block's number, that is by the column, as before by the cut.
-  const int rotation = __builtin_amdgcn_readfirstlane(slabs == 1 ? (int)((blockIdx.x * 37u) % (unsigned)steps) : 0);
   const uint32_t lds0 = (uint32_t)(uintptr_t)(&lds[0]);
   auto issue = [&](int buf) {
-    int k_step = i_step + rotation;  // where along K this step reads
+    int k_step = __builtin_amdgcn_readfirstlane(i_step + rotation);  // where along K this step reads (uniform)
     if (k_step >= steps) k_step -= steps;
     const bf16_t* ws = wsrc + (size_t)k_step * TL_BK;
     const bf16_t* as = asrc + (size_t)k_step * TL_BK;
