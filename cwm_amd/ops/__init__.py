@@ -187,15 +187,13 @@ def gate_up_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
     fused = (
         grouped and n % 16 == 0
         and x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-        and x.shape[0] <= 16 and _stream_takes(x, weight)
+        and x.shape[0] <= STREAM_EPILOGUE_ROWS and _stream_takes(x, weight)
         and (x.shape[1] + 31) // 32 <= 16 * 12  # K fits one group of wavefronts: no split
     )
-    if fused:
+    tiled = x.is_cuda and x.dim() == 2 and _prefers_tile(x, weight, bias)
+    if fused and not tiled:
         return gemm_bf16_stream(x, weight, bias, torch.bfloat16, glu=True)
-    if (
-        grouped and bias is None and x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-        and STREAM_FUSED_ROWS < x.shape[0] <= TILE_ROWS and _tile_takes(x, weight)
-    ):
+    if tiled and grouped and x.shape[0] <= TILE_ROWS:
         return gemm_bf16_tile(x, weight, None, torch.bfloat16, glu=True)
     return silu_mul(linear(x, weight, bias, partials_ok=True), out_dtype=x.dtype, grouped=grouped)
 
@@ -438,10 +436,11 @@ def qkv_rope_write(
     fused = (
         x.is_cuda
         and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16
-        and x.shape[0] <= 16
+        and x.shape[0] <= STREAM_EPILOGUE_ROWS
         and head_dim <= 256
         and _stream_takes(x, weight)
         and (x.shape[1] + 31) // 32 <= 16 * 12  # K fits one group of wavefronts: no split
+        and not _prefers_tile(x, weight, bias)
     )
     if fused:
         _i32(positions, "positions")
@@ -606,9 +605,18 @@ def gemm_bf16_tile(
     return out if out.dim() == 3 or out.dtype == out_dtype else out.to(out_dtype)
 
 
-STREAM_FUSED_ROWS = 16  # rows up to which the streaming product keeps x in registers and has every epilogue
+# rows up to which the streaming product (x in registers, every epilogue in the kernel) is preferred; its epilogues take
+# up to 16, but from 9 on the tiled product is as fast or faster where it takes the sizes (a decode step of the 32B shape at
+# batch 16: 15.3 against 15.6 ms)
+STREAM_FUSED_ROWS = 8
+STREAM_EPILOGUE_ROWS = 16
 TILE_ROWS = 128  # rows up to which the tiled product reads W once
 TILE_ROWS_SHARED = 256  # rows up to which it still beats the library where blocks share tiles (a narrow result)
+
+
+def _prefers_tile(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> bool:
+    """Whether this product goes to the tiled kernel (which has no bias of its own)."""
+    return x.shape[0] > STREAM_FUSED_ROWS and bias is None and _tile_wins(x, weight)
 
 
 def _tile_wins(x: torch.Tensor, weight: torch.Tensor) -> bool:
@@ -648,7 +656,7 @@ def gemm_bf16(
 ) -> torch.Tensor:
     """bfloat16 x [M, K] @ bfloat16 weight[N, K]^T, float32 accumulation.
 
-    Up to 16 rows: the hand-written persistent weight-streaming kernel, x in registers.
+    Up to 8 rows: the hand-written persistent weight-streaming kernel, x in registers.
     Up to 128 rows (256 for a narrow result): the hand-written tiled kernel, x and W
     through LDS (it needs K % 64 == 0 and N % 16 == 0; other sizes of up to 64 rows stream).
     More rows: the library product (hipBLASLt through torch), as the reference calls a
@@ -660,7 +668,7 @@ def gemm_bf16(
     m = x.shape[0]
     if not _stream_takes(x, weight):
         return gemm_f32(x, weight, bias, out_dtype)
-    if m > STREAM_FUSED_ROWS and bias is None and _tile_wins(x, weight):  # (the tiled kernel has no bias of its own)
+    if _prefers_tile(x, weight, bias):
         return gemm_bf16_tile(x, weight, None, out_dtype, partials_ok)
     if m <= STREAM_MAX_ROWS:
         return gemm_bf16_stream(x, weight, bias, out_dtype, partials_ok)

@@ -935,7 +935,7 @@ def test_gemm_bf16_tile_gated_epilogue(m, f, k, units):
     torch.testing.assert_close(fused.cpu().double(), want, rtol=3e-2, atol=3e-2 * float(want.abs().max()))
 
 
-def test_products_of_17_to_128_rows_take_the_tiled_kernel():
+def test_products_of_9_to_128_rows_take_the_tiled_kernel():
     """`linear` and `gate_up_silu` route the sizes the tiled kernel takes to it, and the others as before."""
     from cwm_amd import ops
 
@@ -948,8 +948,12 @@ def test_products_of_17_to_128_rows_take_the_tiled_kernel():
     assert torch.equal(ops.linear(xo, odd), ops.gemm_bf16_stream(xo, odd))
     with pytest.raises(ops.KernelError, match="tiled product takes"):
         ops.gemm_bf16_tile(xo, odd)
-    x16 = x[:16].contiguous()
-    assert torch.equal(ops.linear(x16, w), ops.gemm_bf16_stream(x16, w))
+    # up to 8 rows the streaming product is preferred; its epilogues serve up to 16 where the tiled kernel refuses
+    x8, x12 = x[:8].contiguous(), x[:12].contiguous()
+    assert torch.equal(ops.linear(x8, w), ops.gemm_bf16_stream(x8, w))
+    assert torch.equal(ops.linear(x12, w), ops.gemm_bf16_tile(x12, w))
+    assert torch.equal(ops.gate_up_silu(x12, w, None, True), ops.gemm_bf16_tile(x12, w, glu=True))
+    assert torch.equal(ops.gate_up_silu(xo[:12].contiguous(), odd, None, True), ops.gemm_bf16_stream(xo[:12].contiguous(), odd, None, torch.bfloat16, glu=True))
 
 
 @pytest.mark.parametrize("n_q,n_kv,hd,page_size,dim,m", [(4, 2, 16, 8, 64, 40), (6, 1, 64, 16, 128, 70), (12, 2, 128, 64, 256, 33), (3, 3, 48, 8, 192, 100)])
