@@ -86,6 +86,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--shape", default="cwm32b", choices=sorted(SHAPES), help="layer sizes; the default is the headline configuration")
+    ap.add_argument("--config", default=None, metavar="FILE", help="a config.json of the architecture whose layer sizes are measured instead of --shape's")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (both numbers are reported)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--batch", type=int, default=8)
@@ -115,6 +116,9 @@ def main() -> int:
 
     device = torch.device("cuda:0")
     shape_name, shape = SHAPES[args.shape]
+    if args.config:
+        with open(args.config) as f:
+            shape_name, shape = f"the sizes of {os.path.basename(args.config)}", json.load(f)
     config = dict(shape)
     full_layers = shape["n_layers"]
     if args.layers is None:

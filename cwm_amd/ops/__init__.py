@@ -6,8 +6,8 @@ no CPU path and no library substitute: tensors that are not on a HIP device, or 
 missing kernel library, raise an error.
 
 The only library routine on the model's path is the bfloat16 matrix product for
-more rows than the hand-written streaming kernel takes (`torch.matmul`, i.e.
-hipBLASLt), where the reference also calls a library
+more rows than the hand-written kernels take (`torch.mm`, i.e. hipBLASLt), where
+the reference also calls a library
 (cwm/fastgen/forward.py:593-606).
 """
 
@@ -399,9 +399,12 @@ def gemm_bf16_stream(
     return out
 
 
+_NO_ROPE_ARGS = [ctypes.c_void_p(0)] * 5 + [ctypes.c_int(0)] * 6
+
+
 def _rope_args(rope: Optional[tuple]) -> list:
     if rope is None:
-        return [ctypes.c_void_p(0)] * 5 + [ctypes.c_int(0)] * 6
+        return _NO_ROPE_ARGS
     positions, seq_of_token, inv_freq, cache, block_table, n_q, n_kv, hd = rope
     return [
         _ptr(positions), _ptr(seq_of_token), _ptr(inv_freq), _ptr(cache), _ptr(block_table),

@@ -194,6 +194,10 @@ def build(name: str, defines: Optional[Mapping[str, int]] = None, force: bool = 
 
 def load(name: str, defines: Optional[Mapping[str, int]] = None) -> ctypes.CDLL:
     """The library of `csrc/<name>.hip`, built first if need be."""
+    if defines is None:
+        lib = _loaded.get(name)  # the common case, on every launch: no lock, no tag
+        if lib is not None:
+            return lib
     key = name + _variant_tag(defines or {})
     with _lock:
         lib = _loaded.get(key)
