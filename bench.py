@@ -93,6 +93,7 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=32768)
     ap.add_argument("--page", type=int, default=256)
     ap.add_argument("--no-points", action="store_true")
+    ap.add_argument("--graphs", type=int, default=16, help="decode steps kept as HIP graphs where the host is the limit, as the engine's default (0: none)")
     ap.add_argument(
         "--serve",
         type=int,
@@ -174,7 +175,7 @@ def main() -> int:
         storage = CacheStorage(manager, device, model.runtime.act_dtype)
         for t in storage.paged.values():
             t.normal_(0.0, 1.0)
-        return ModelRunner(model, manager, storage), manager
+        return ModelRunner(model, manager, storage, num_graphs=args.graphs, graphs_where_host_bound=True), manager
 
     def decode_run(batch, ctx, steps, warmup):
         """tokens/s and ms per step of `steps` decode steps of `batch` requests that

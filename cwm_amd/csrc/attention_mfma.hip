@@ -147,6 +147,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __res
   const int key_begin = w[2];
   const int key_end = w[3];
   const int slot = w[4];
+  if (key_begin >= key_end) return;  // a null item: a list of a fixed length is filled up with them
 
   const int group = n_q_heads / n_kv_heads;
   const int q0 = cu_q[b];

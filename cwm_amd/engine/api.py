@@ -28,7 +28,8 @@ class GenArgs:
     max_gen: Optional[int] = None  # most new tokens of a request
 
     host_cache_gb: float = 0  # host prefix cache: not built, must be 0
-    num_cuda_graphs: int = 16  # decode graph buckets of the reference: ignored
+    num_cuda_graphs: int = 16  # decode steps kept as HIP graphs, one per number of requests (the reference: one per bucket of
+    # batch sizes); 0, or FG_NO_CUDA_GRAPHS in the environment: every step is launched kernel by kernel
     cache_block: int = 256  # tokens in a page
     max_prefill: int = 4096  # token budget of one step
     min_prefill: int = 512  # reference batching threshold: not needed with mixed steps, ignored

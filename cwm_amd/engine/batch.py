@@ -48,6 +48,7 @@ class StepBatch:
     rids: List[Hashable] = field(default_factory=list)
     page_size: int = 0
     scratch: Dict[Any, Any] = field(default_factory=dict)  # per-step plans that kernels' wrappers keep
+    static: Any = None  # for a step that is captured and replayed: the fixed homes of such plans (`ops.StaticPlans`)
 
     @property
     def max_q_len(self) -> int:
@@ -68,11 +69,17 @@ def build_batch(
     device: torch.device,
     vocab_size: int,
     tokens_device: Optional[torch.Tensor] = None,
+    table_width: Optional[int] = None,
+    into: Optional[torch.Tensor] = None,
 ) -> StepBatch:
     """Descriptor for `portions`; the pages of their tokens must already be held
     (`CacheManager.extend`).  `tokens_device` (int32 [T] on the device) takes the place of the
     portions' token ids, which then only count: a decode step whose tokens the step before has
-    sampled and which have not been to the host."""
+    sampled and which have not been to the host.  `table_width`: columns of the block tables (at
+    least what the longest sequence needs; the rest holds -1).  `into`: an int32 vector on the
+    device that receives the descriptor instead of a new one, so that steps of one shape (the same
+    numbers of tokens, sequences, wanted rows and table columns) have their vectors at the same
+    addresses."""
     if not portions:
         raise BatchError("a step needs at least one portion")
     n_seqs = len(portions)
@@ -119,6 +126,10 @@ def build_batch(
 
     page_size = manager.page_size
     width = max(1, max((kv + page_size - 1) // page_size for kv in kv_lens))
+    if table_width is not None:
+        if table_width < width:
+            raise BatchError(f"block tables of {table_width} columns do not hold the {width} pages of the longest sequence")
+        width = table_width
     tables = []
     columns = np.arange(width, dtype=np.int64)[None, :]
     last_page = np.asarray([pages_for(kv, page_size) for kv in kv_lens], dtype=np.int64)[:, None]
@@ -163,7 +174,13 @@ def build_batch(
     host_np = host.numpy()
     for off, seg in zip(offsets, segments):
         host_np[off : off + seg.size] = seg
-    dev = host.to(device, non_blocking=use_pinned)
+    if into is None:
+        dev = host.to(device, non_blocking=use_pinned)
+    else:
+        if into.dtype != torch.int32 or into.dim() != 1 or into.numel() < host.numel() or into.device.type != device.type:
+            raise BatchError(f"the descriptor's {host.numel()} numbers do not fit the vector given for them")
+        dev = into
+        dev[: host.numel()].copy_(host, non_blocking=use_pinned)
 
     def seg(i: int) -> torch.Tensor:
         return dev[offsets[i] : offsets[i] + segments[i].size]

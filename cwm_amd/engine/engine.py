@@ -137,7 +137,12 @@ class Engine:
         sizes = pool_sizes(model, args, self.device)
         self.manager = CacheManager(model.cache_specs, args.cache_block, sizes, args.max_batch)
         self.storage = CacheStorage(self.manager, self.device, model.runtime.act_dtype)
-        self.runner = ModelRunner(model, self.manager, self.storage)
+        # decode steps as graphs, one per number of requests (the reference captures one per bucket of batch sizes and
+        # pads, cwm/fastgen/generate.py:313-373, and has the same switch to go without)
+        use_graphs = not os.environ.get("FG_NO_CUDA_GRAPHS")
+        self.runner = ModelRunner(
+            model, self.manager, self.storage, num_graphs=max(0, args.num_cuda_graphs) if use_graphs else 0, graphs_where_host_bound=True
+        )
         # a request joins others only when its known tokens and some room to decode fit
         # (the reference asks for 128 tokens of room, cwm/fastgen/generate.py:596-597)
         self.scheduler = Scheduler(self.manager, args.max_batch, args.max_prefill, headroom=min(128, args.cache_block))

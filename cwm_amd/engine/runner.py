@@ -10,18 +10,47 @@ them in one call (cwm/fastgen/generate.py:480-498).
 
 from __future__ import annotations
 
-from typing import Callable, Hashable, List, Optional, Sequence
+import sys
+from collections import OrderedDict
+from dataclasses import dataclass
+from typing import Any, Callable, Hashable, List, Optional, Sequence
 
 import torch
 
 from ..cache.manager import CacheManager
+from ..cache.pages import pages_for
 from ..cache.storage import CacheStorage
 from ..models.model import Model
-from .batch import Portion, build_batch
+from .batch import Portion, StepBatch, build_batch
+
+
+@dataclass
+class CapturedStep:
+    """A decode step of `n_seqs` requests as a HIP graph, with what it reads and writes at fixed addresses
+    (the reference's DecodeGraph, cwm/fastgen/generate.py:71-75,339-373)."""
+
+    graph: Any  # torch.cuda.CUDAGraph
+    descriptor: torch.Tensor  # the step's descriptor (int32), filled anew before every replay
+    table_width: int  # columns of its block tables: the sequences may grow to that many pages
+    plans: Any  # ops.StaticPlans: the kernels' work lists, likewise
+    tokens: torch.Tensor  # the descriptor's token ids
+    logits: torch.Tensor  # where a replay leaves its logits
 
 
 class ModelRunner:
-    def __init__(self, model: Model, manager: CacheManager, storage: CacheStorage) -> None:
+    # a step is worth a capture when the host took at least this share of the step's time to launch it
+    HOST_BOUND_SHARE = 0.85
+
+    def __init__(
+        self, model: Model, manager: CacheManager, storage: CacheStorage, num_graphs: int = 0, graphs_where_host_bound: bool = False
+    ) -> None:
+        """`num_graphs`: decode steps (one token of every request, the logits of all wanted) are captured as
+        HIP graphs, one per number of requests, and replayed, which spares the host the launch of every
+        kernel; at most so many are kept, the least recently used goes.  0, a model some part of which is
+        not `replayable`, or a device that is no GPU: every step is launched kernel by kernel.
+        `graphs_where_host_bound`: a number of requests gets its capture only if launching its step keeps
+        the host busy for most of the step's time (measured on its second and third step; where the GPU's
+        time is the longer one a replay gains nothing, and its lists of a fixed length cost a little)."""
         if model.runtime is None:
             raise RuntimeError("the model has no weights yet (Model.bind)")
         self.model = model
@@ -30,6 +59,13 @@ class ModelRunner:
         self.device = model.runtime.device
         # called as on_pages_freed(group, pages) whenever pages go back to a pool
         self.on_pages_freed: Optional[Callable[[int, List[int]], None]] = None
+        self.num_graphs = num_graphs if self.device.type == "cuda" and model.replayable else 0
+        self.graphs_where_host_bound = graphs_where_host_bound
+        self._host_share: dict = {}  # number of requests -> shares of the step's time that the host spent launching it
+        self._captured: "OrderedDict[int, CapturedStep]" = OrderedDict()
+        self._graph_pool: Any = None
+        self.n_captures = 0
+        self.n_replays = 0
 
     # ---- requests ------------------------------------------------------------- #
     def admit(self, rid: Hashable) -> int:
@@ -55,8 +91,89 @@ class ModelRunner:
         place is wanted.  Afterwards every request's length has grown by its portion
         and window groups have given back the pages that fell out of reach.  With
         `tokens_device` the token ids come from that device tensor (see `build_batch`)."""
-        batch = build_batch(portions, self.manager, self.device, self.model.vocab_size, tokens_device)
-        logits = self.model.forward(batch, self.storage)
+        if (
+            self.num_graphs > 0 and portions
+            and all(len(p.tokens) == 1 and len(p.want) == 1 and p.want[0] == 0 and p.rid in self.manager for p in portions)
+        ):
+            logits = self._decode_step(portions, tokens_device)
+        else:
+            batch = build_batch(portions, self.manager, self.device, self.model.vocab_size, tokens_device)
+            logits = self.model.forward(batch, self.storage)
         for portion in portions:
             self._report(self.manager.advance(portion.rid, len(portion.tokens)))
         return logits
+
+    # ---- decode steps as graphs ---------------------------------------------------- #
+    def _decode_step(self, portions: Sequence[Portion], tokens_device: Optional[torch.Tensor]) -> torch.Tensor:
+        """A step of one token per request: the replay of its capture if there is one that still holds it,
+        else the step itself, launched kernel by kernel, and then its capture for the steps to come."""
+        n = len(portions)
+        page = self.manager.page_size
+        width = max(pages_for(self.manager.length(p.rid) + 1, page) for p in portions)
+        held = self._captured.get(n)
+        if held is not None and width <= held.table_width:
+            batch = self._static_batch(portions, held.descriptor, held.table_width, held.plans, tokens_device)
+            if held.plans.refresh(batch):
+                held.graph.replay()
+                self._captured.move_to_end(n)
+                self.n_replays += 1
+                return held.logits.clone()  # the next replay writes there again
+        self._captured.pop(n, None)  # outgrown: its tables or work lists have no room for this step
+        if self.graphs_where_host_bound and not self._worth_a_capture(n):
+            return self._launched_and_timed(portions, tokens_device, n)
+        table_width = width + max(width // 4, 2)
+        n_groups = len(self.manager.groups)
+        descriptor = torch.empty(8 * (n + 4) + n_groups * (n * table_width + 4), dtype=torch.int32, device=self.device)
+        from .. import ops
+
+        plans = ops.StaticPlans(self.device, max_keys=table_width * page)
+        batch = self._static_batch(portions, descriptor, table_width, plans, tokens_device)
+        logits = self.model.forward(batch, self.storage)  # this step; the work lists find their homes in it
+        try:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                static_logits = self.model.forward(batch, self.storage)
+        except Exception as exc:  # the step above has run and stands; later ones are launched kernel by kernel
+            print(f"[cwm_amd] decode steps are not captured as graphs: {type(exc).__name__}: {exc}", file=sys.stderr, flush=True)
+            self.num_graphs = 0
+            self._captured.clear()
+            return logits
+        if self._graph_pool is None:
+            self._graph_pool = graph.pool()
+        self._captured[n] = CapturedStep(graph, descriptor, table_width, plans, batch.tokens, static_logits)
+        self.n_captures += 1
+        while len(self._captured) > self.num_graphs:
+            self._captured.popitem(last=False)
+        return logits
+
+    def _worth_a_capture(self, n: int) -> bool:
+        shares = self._host_share.get(n, ())
+        return len(shares) >= 3 and min(shares[1:3]) >= self.HOST_BOUND_SHARE
+
+    def _launched_and_timed(self, portions: Sequence[Portion], tokens_device: Optional[torch.Tensor], n: int) -> torch.Tensor:
+        """The step, launched kernel by kernel; the first three such steps of `n` requests are timed, on the
+        host and on the device (the first one of them may load libraries and does not count)."""
+        import time
+
+        shares = self._host_share.setdefault(n, [])
+        batch = build_batch(portions, self.manager, self.device, self.model.vocab_size, tokens_device)
+        if len(shares) >= 3:
+            return self.model.forward(batch, self.storage)
+        torch.cuda.synchronize(self.device)
+        start = time.perf_counter()
+        logits = self.model.forward(batch, self.storage)
+        launched = time.perf_counter() - start
+        torch.cuda.synchronize(self.device)
+        shares.append(launched / max(time.perf_counter() - start, 1e-9))
+        return logits
+
+    def _static_batch(
+        self, portions: Sequence[Portion], descriptor: torch.Tensor, table_width: int, plans: Any, tokens_device: Optional[torch.Tensor]
+    ) -> StepBatch:
+        batch = build_batch(portions, self.manager, self.device, self.model.vocab_size, None, table_width, descriptor)
+        batch.static = plans
+        if tokens_device is not None:
+            if tokens_device.dtype != torch.int32 or tokens_device.numel() != batch.n_tokens:
+                raise ValueError(f"tokens on the device must be int32 [{batch.n_tokens}]")
+            batch.tokens.copy_(tokens_device.reshape(-1))
+        return batch

@@ -83,6 +83,11 @@ class Model:
         prefix = plan.final_norm_name + "."
         self.final_norm.bind({n[len(prefix):]: t for n, t in tensors.items() if n.startswith(prefix)}, runtime)
 
+    @property
+    def replayable(self) -> bool:
+        """Whether a decode step may be captured once and replayed: every part says so (`Part.replayable`)."""
+        return all(block.replayable for block in self.blocks) and self.final_norm.replayable
+
     # ---- one step ------------------------------------------------------------------ #
     def forward(self, batch, cache) -> Optional[torch.Tensor]:
         """Run the batch's tokens through every layer, writing the cache, and return

@@ -818,10 +818,61 @@ class _UploadedPlan:
     wide_shape: Tuple[int, float]  # key tiles of the longest wide item, and the mean
 
 
+class StaticPlans:
+    """The attention work lists of a step that is captured once and replayed: every list has a home of a
+    fixed size at a fixed address, which `refresh` fills for each new step (unused places hold null items),
+    so that the captured launches stay valid while the sequences grow.  The first, uncaptured run of the step
+    finds out which lists the model's layers ask for and makes their homes."""
+
+    def __init__(self, device: torch.device, max_keys: int) -> None:
+        self.device = device
+        self.max_keys = max_keys  # the most keys a sequence may hold while the capture is in use
+        self.homes: dict = {}  # (group, key/value heads, window) -> (capacity, device vector, uploaded plan)
+
+    def _padded(self, batch, group: int, n_kv: int, window: Optional[int], capacity):
+        from .attention_plan import PlanCapacity, build_plan, pad_plan
+
+        wide_cut_below = -(-2 * _compute_units(self.device) // n_kv)
+        plan = build_plan(batch.q_lens, batch.kv_lens, group, window, wide_cut_below)
+        if capacity is None:
+            capacity = PlanCapacity.roomy(plan)
+        flat = pad_plan(plan, capacity)
+        return plan, capacity, flat
+
+    def plan(self, batch, group: int, n_kv: int, window: Optional[int]) -> "_UploadedPlan":
+        key = (group, n_kv, window)
+        home = self.homes.get(key)
+        if home is None:
+            plan, capacity, flat = self._padded(batch, group, n_kv, window, None)
+            if flat is None:
+                raise KernelError("this step's attention work has items that a captured step does not take")
+            dev = torch.from_numpy(flat).pin_memory().to(self.device, non_blocking=True)
+            a = capacity.work * 6
+            uploaded = _UploadedPlan(
+                work=dev[:a], wide=dev[a:a], merge=dev[a:], n_work=capacity.work, n_wide=0, n_merge=capacity.merge,
+                n_merge_mid=capacity.merge_mid, n_merge_wide=0, n_partials=capacity.work,
+                work_keys=int((plan.work[:, 3] - plan.work[:, 2]).mean()) if plan.work.shape[0] else 0, wide_shape=(0, 0.0),
+            )
+            home = self.homes[key] = (capacity, dev, uploaded)
+        return home[2]
+
+    def refresh(self, batch) -> bool:
+        """Fill every home with the lists of `batch`; False if one of them has outgrown its home."""
+        for (group, n_kv, window), (capacity, dev, _) in self.homes.items():
+            _, _, flat = self._padded(batch, group, n_kv, window, capacity)
+            if flat is None:
+                return False
+            dev.copy_(torch.from_numpy(flat).pin_memory(), non_blocking=True)
+        return True
+
+
 def _attention_plan(batch, group: int, n_kv: int, window: Optional[int], device: torch.device) -> _UploadedPlan:
     """The step's work list for this (group size, key/value heads, window), uploaded once per step."""
     from .attention_plan import build_plan
 
+    static = getattr(batch, "static", None)
+    if static is not None:
+        return static.plan(batch, group, n_kv, window)
     key = ("attention_plan", group, n_kv, window)
     cached = batch.scratch.get(key)
     if cached is None:
@@ -941,7 +992,9 @@ def paged_attention(
     hd = q.shape[2]
     if q.is_cuda and mfma_attention_takes(q.dtype, hd, cache.shape[3] // hd):
         return paged_attention_mfma(q, cache, block_table, batch, window, scale)
-    return paged_attention_simple(q, cache, block_table, batch.positions, batch.seq_of_token, window, scale, max_keys=batch.max_kv_len)
+    static = getattr(batch, "static", None)
+    max_keys = batch.max_kv_len if static is None else static.max_keys
+    return paged_attention_simple(q, cache, block_table, batch.positions, batch.seq_of_token, window, scale, max_keys=max_keys)
 
 
 # --------------------------------------------------------------------------- #

@@ -171,3 +171,56 @@ def _tile_ranges(n_new: int, kv: int, n_tiles: int, group: int, window: Optional
     key_hi = n_old + last_tok + 1  # exclusive
     key_lo = np.zeros_like(row0) if window is None else np.maximum(0, n_old + first_tok - (window - 1))
     return key_lo, key_hi, row0
+
+
+# an item that no kernel acts on: its first row lies beyond every sequence's rows and it names no key
+NULL_ROW = 1 << 24
+NULL_WORK = (0, NULL_ROW, 0, 0, -1, 0)
+NULL_MERGE = (0, NULL_ROW, 0, 0)
+
+
+@dataclass(frozen=True)
+class PlanCapacity:
+    """Sizes of a plan's lists that do not change from step to step: a captured step launches these many
+    items whatever the step holds, and the unused ones are null items."""
+
+    work: int
+    merge_many: int
+    merge_mid: int
+
+    @property
+    def merge(self) -> int:
+        return self.merge_many + self.merge_mid
+
+    @property
+    def ints(self) -> int:
+        return self.work * WORK_INTS + self.merge * 4
+
+    @staticmethod
+    def roomy(plan: AttentionPlan) -> "PlanCapacity":
+        """Room for `plan` and for a quarter more keys: every tile's keys grow, so a tile that is not yet cut
+        will be, each gains a chunk now and then, and a merge item whose partials come near MERGE_MID_MAX will
+        move from the items of few partials to those of many (no item is near: no launch for those at all)."""
+        tiles = int((plan.work[:, 4] < 0).sum()) + plan.merge.shape[0]
+        work = plan.work.shape[0]
+        near_many = int((plan.merge[:, 3] > (3 * MERGE_MID_MAX) // 4).sum())
+        many_now = plan.merge.shape[0] - plan.n_merge_mid - plan.n_merge_wide
+        return PlanCapacity(work=work + max(work // 4, 2 * tiles, 16), merge_many=near_many, merge_mid=tiles - many_now)
+
+
+def pad_plan(plan: AttentionPlan, capacity: PlanCapacity) -> Optional[np.ndarray]:
+    """`plan` as one int32 vector of `capacity.ints` numbers: the work items, then the merge items of many
+    partials, then those of few, each list filled up with null items.  None if the plan does not fit, or has
+    items that a captured step does not take (blocks of many rows)."""
+    n_merge = plan.merge.shape[0]
+    n_many = n_merge - plan.n_merge_mid - plan.n_merge_wide
+    if plan.work_wide.shape[0] or plan.n_merge_wide:
+        return None
+    if plan.work.shape[0] > capacity.work or n_many > capacity.merge_many or plan.n_merge_mid > capacity.merge_mid:
+        return None
+    work = np.tile(np.asarray(NULL_WORK, dtype=np.int32), (capacity.work, 1))
+    work[: plan.work.shape[0]] = plan.work
+    merge = np.tile(np.asarray(NULL_MERGE, dtype=np.int32), (capacity.merge, 1))
+    merge[:n_many] = plan.merge[:n_many]
+    merge[capacity.merge_many : capacity.merge_many + plan.n_merge_mid] = plan.merge[n_many:]
+    return np.concatenate([work.reshape(-1), merge.reshape(-1)])

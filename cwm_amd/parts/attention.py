@@ -101,7 +101,15 @@ class PagedAttention(Mixer):
         """The seam between projection and rotation: a subclass may change the projected queries
         `q` [T, Hq, hd] and keys `k` [T, Hkv, hd] (None when this call writes no cache) in place
         here (a norm per head, say) before they are rotated and the keys are cached.  Overriding it
-        takes the step off the fused projection + rotation + cache-write kernel."""
+        takes the step off the fused projection + rotation + cache-write kernel, and off captured
+        steps unless the subclass sets `transform_replayable`."""
+
+    transform_replayable = False  # whether an overriding `transform_qk` keeps to the rule of `Part.replayable`
+
+    @property
+    def replayable(self) -> bool:
+        own = type(self).transform_qk is PagedAttention.transform_qk or self.transform_replayable
+        return own and (self.position_encoding is None or self.position_encoding.replayable)
 
     def forward(self, x: torch.Tensor, batch: Any, cache: Any, write_cache: bool = True) -> torch.Tensor:
         hd = self.head_dim

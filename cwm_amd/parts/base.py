@@ -106,6 +106,13 @@ class Runtime:
 class Part:
     """Base of every part."""
 
+    # Whether a decode step through this part may be captured once and replayed: its `forward` then launches
+    # the same kernels with the same arguments for every step of that shape, and reads what changes from step
+    # to step (tokens, positions, lengths, block tables, state slots) from the step's device vectors only;
+    # nothing goes between host and device in it.  A part that does not say so keeps its model on the path
+    # that launches every step kernel by kernel.
+    replayable = False
+
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         return {}
 

@@ -24,6 +24,10 @@ class PreNormBlock(Block):
         self.names = dict(names)
         self._parts = {"norm1": norm1, "mixer": mixer, "norm2": norm2, "feed_forward": feed_forward}
 
+    @property
+    def replayable(self) -> bool:
+        return all(part.replayable for part in self._parts.values())
+
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         specs: Dict[str, TensorSpec] = {}
         for role, part in self._parts.items():

@@ -17,6 +17,8 @@ class SwiGLU(FeedForward):
     gate's SiLU and the product with the up branch are computed in float32 and
     rounded once."""
 
+    replayable = True
+
     def __init__(self, dim: int, hidden_dim: int) -> None:
         self.dim = dim
         self.hidden_dim = hidden_dim

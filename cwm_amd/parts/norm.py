@@ -16,6 +16,8 @@ class RMSNorm(Norm):
     772,789).  The residual update that the reference adds just before
     (`h.add_`, forward.py:769,786) is added here, in float32, in the same kernel."""
 
+    replayable = True
+
     def __init__(self, dim: int, eps: float) -> None:
         self.dim = dim
         self.eps = float(eps)

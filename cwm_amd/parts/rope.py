@@ -49,6 +49,8 @@ class RotaryEncoding(PositionEncoding):
     position * inv_freq[i] (cwm/fastgen/kernels/rope.py:55-90).  The table is all a
     kernel needs; a scaling scheme only changes the table."""
 
+    replayable = True
+
     def __init__(self, head_dim: int, theta: float, llama3_scaling: Optional[Mapping[str, float]] = None) -> None:
         if head_dim % 2 != 0:
             raise ValueError("rotary pairs need an even head size")
@@ -77,6 +79,8 @@ class RotaryEncoding(PositionEncoding):
 
 class NoPositionEncoding(PositionEncoding):
     """Queries and keys are used as they are."""
+
+    replayable = True
 
 
 register_part("position_encoding", "rotary", RotaryEncoding)

@@ -23,7 +23,10 @@ partly filled beyond its multiple of 64); `--pages all=N,8192=M` sets the pools'
 pages outright, by the group's window (`all`: the group that keeps every key);
 `--random-config FILE --seed S [--std X]` runs the configuration in FILE with random
 weights instead of a model folder; `--page-log FILE` writes, per step, the pages every
-request took and the pages that went back to each group's pool, as JSON lines.
+request took and the pages that went back to each group's pool, as JSON lines;
+`--graphs N` runs steps of single tokens whose logits are all wanted as generation does by
+default: captured as HIP graphs, one per number of requests and at most N of them, and
+replayed (default 0: every step is launched kernel by kernel).
 
 The reference has no such tool; its nearest hooks are prompt log-probabilities
 (cwm/fastgen/forward.py:908-924) and the eager decode path
@@ -65,6 +68,7 @@ class Replayer:
         seed: int = 0,
         std: float = 0.02,
         page_log: Optional[str] = None,
+        num_graphs: int = 0,
     ) -> None:
         from .cache import CacheManager, CacheStorage
         from .engine import ModelRunner, load_model, random_model
@@ -95,7 +99,7 @@ class Replayer:
                 raise ValueError(f"--pages names groups that the model does not have: {sorted(map(str, unknown))}; its groups: {sorted(map(str, sizes))}")
         self.manager = CacheManager(self.model.cache_specs, page_size, sizes, max_requests)
         self.storage = CacheStorage(self.manager, self.device, self.model.runtime.act_dtype)
-        self.runner = ModelRunner(self.model, self.manager, self.storage)
+        self.runner = ModelRunner(self.model, self.manager, self.storage, num_graphs=num_graphs)
         self.poison_freed_pages = poison_freed_pages
         self._given: Dict[int, List[int]] = {}
         self._log = open(page_log, "w", encoding="utf-8") if page_log else None
@@ -167,6 +171,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     parser.add_argument("--seed", type=int, default=0, help="seed of those random weights")
     parser.add_argument("--std", type=float, default=0.02, help="standard deviation of those random weights")
     parser.add_argument("--page-log", help="file that receives the pages taken and given back, one JSON line a step")
+    parser.add_argument("--graphs", type=int, default=0, help="decode steps kept as HIP graphs (0: none)")
     args = parser.parse_args(argv)
     if (args.model is None) == (args.random_config is None):
         parser.error("give exactly one of --model and --random-config")
@@ -184,7 +189,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     os.makedirs(args.out, exist_ok=True)
     replayer = Replayer(
         args.model, args.dtype, args.max_tokens, device=args.device, page_size=args.page_size, pages=pages,
-        random_config=random_config, seed=args.seed, std=args.std, page_log=args.page_log,
+        random_config=random_config, seed=args.seed, std=args.std, page_log=args.page_log, num_graphs=args.graphs,
     )
     for line in sys.stdin:
         line = line.strip()

@@ -1,0 +1,119 @@
+"""Decode steps that are captured as HIP graphs and replayed, against the same steps launched kernel by
+kernel and against the plain implementation: through the replay driver (tails decoded one by one, mixed
+steps between them, pages given back and used again, sequences that outgrow a capture) and through the
+engine (greedy and sampled generation)."""
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import compare as cmp, configs, models, traces
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = tmp_path_factory.mktemp("models")
+    return {(name, dtype): models.make_folder(root, name, seed=11, dtype=dtype) for name in ("tiny_a", "tiny_b", "tiny_d") for dtype in ("float32", "bfloat16")}
+
+
+def decode_steps(requests, tail):
+    """Everything but the last `tail` tokens of each request in one step, then one token of every request a
+    step; the shortest request ends first, so the steps see a falling number of requests."""
+    steps = [{"step": 0, "entries": [{"id": rid, "tokens": toks[:-tail], "want": list(range(len(toks) - tail))} for rid, toks in requests.items()], "end": []}]
+    done = {rid: len(toks) - tail for rid, toks in requests.items()}
+    live = list(requests)
+    while live:
+        entries = []
+        for rid in live:
+            entries.append({"id": rid, "tokens": [requests[rid][done[rid]]], "want": [0]})
+            done[rid] += 1
+        end = [rid for rid in live if done[rid] == len(requests[rid])]
+        steps.append({"step": len(steps), "entries": entries, "end": end})
+        live = [rid for rid in live if rid not in end]
+    return steps
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["tiny_a", "tiny_b", "tiny_d"])
+def test_replayed_steps_give_the_logits_of_launched_ones(folders, name, dtype):
+    """150 and more single-token steps of up to four requests, across many pages, chunks of keys and (tiny_b,
+    tiny_d) the window, with pages that go back to the pool and are poisoned: the logits of every step are
+    those of the run without graphs, bit for bit, and those of the plain implementation within the limits;
+    a capture serves many steps."""
+    from cwm_amd.replay import Replayer
+
+    vocab = configs.get(name)["vocab_size"]
+    lengths = [260, 200, 171, 333]
+    requests = {f"r{i}": traces.random_tokens(31 * i + 5, n, vocab) for i, n in enumerate(lengths)}
+    steps = decode_steps(requests, tail=150)
+    max_tokens = traces.max_live_tokens(steps)
+    page_size = 32 if name == "tiny_d" else 8
+    outputs = {}
+    for graphs in (0, 4):
+        rep = Replayer(folders[name, dtype], dtype, max_tokens, page_size=page_size, poison_freed_pages=True, num_graphs=graphs)
+        outputs[graphs] = traces.run_in_process(rep, steps)
+        if graphs:
+            assert rep.runner.n_replays > 100 and rep.runner.n_captures <= 24, (rep.runner.n_replays, rep.runner.n_captures)
+        assert rep.manager.live_requests() == []
+    for step, want in outputs[0].items():
+        assert np.array_equal(outputs[4][step], want), f"step {step} differs between the replayed and the launched run"
+    got = traces.gather(steps, outputs[4], {k: len(v) for k, v in requests.items()}, vocab)
+    want = cmp.expected(folders[name, dtype], requests, dtype)
+    for rid in requests:
+        cmp.check(got[rid], want[rid], dtype, f"{name} {dtype} graphs {rid}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixed_steps_between_replays(folders, dtype):
+    """Up to four live requests, portions of prompts beside decoded tokens and steps of decoded tokens only
+    (which are replayed) in turn, with so few pages that they are used again: the plain implementation's
+    logits within the limits, and bit for bit those of the run without graphs."""
+    from cwm_amd.replay import Replayer
+
+    name = "tiny_b"
+    vocab = configs.get(name)["vocab_size"]
+    requests = {f"r{i}": traces.random_tokens(3 * i + 1, n, vocab) for i, n in enumerate([9, 40, 100, 57, 230, 77])}
+    steps = traces.mixed(requests, decode_tail=40)
+    max_tokens = traces.max_live_tokens(steps)
+    outputs = {}
+    for graphs in (0, 3):
+        rep = Replayer(folders[name, dtype], dtype, max_tokens, page_size=4, poison_freed_pages=True, num_graphs=graphs)
+        outputs[graphs] = traces.run_in_process(rep, steps)
+        if graphs:
+            assert rep.runner.n_replays > 5, (rep.runner.n_replays, rep.runner.n_captures)
+    for step, out in outputs[0].items():
+        assert np.array_equal(outputs[3][step], out), f"step {step} differs between the replayed and the launched run"
+    got = traces.gather(steps, outputs[3], {k: len(v) for k, v in requests.items()}, vocab)
+    want = cmp.expected(folders[name, dtype], requests, dtype)
+    for rid in requests:
+        cmp.check(got[rid], want[rid], dtype, f"{name} {dtype} mixed with graphs {rid}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_generation_with_and_without_graphs(folders, dtype, monkeypatch):
+    """Greedy and sampled generation of requests that come and go (so the number of decoding requests changes,
+    and bursts of decode steps feed each other on the device): the same tokens and log-probabilities with decode
+    steps replayed from graphs (the default), with two graphs only, and with none."""
+    from cwm_amd.engine import Engine, GenArgs
+
+    name = "tiny_b"
+    vocab = configs.get(name)["vocab_size"]
+    prompts = [traces.random_tokens(70 + i, n, vocab) for i, n in enumerate([5, 33, 64, 90, 12, 41])]
+    results = {}
+    for label, graphs, env in (("default", 16, None), ("two", 2, None), ("none", 0, None), ("switch", 16, "1")):
+        if env is None:
+            monkeypatch.delenv("FG_NO_CUDA_GRAPHS", raising=False)
+        else:
+            monkeypatch.setenv("FG_NO_CUDA_GRAPHS", env)
+        for sampling in (False, True):
+            args = GenArgs(use_sampling=sampling, temperature=0.8, top_p=0.9, max_batch=4, max_seq=4096, cache_block=8, max_prefill=64,
+                           logprobs=True, num_cuda_graphs=graphs, sync_freq=5)
+            engine = Engine.from_folder(folders[name, dtype], args, dtype=dtype)
+            results[label, sampling] = engine.generate_tokens(prompts, max_gen=60)
+            replays = engine.runner.n_replays
+            assert (replays > 0) == (label in ("default", "two")), (label, replays)
+    for sampling in (False, True):
+        for label in ("two", "none", "switch"):
+            assert results[label, sampling] == results["default", sampling], f"{label}, sampling {sampling}"
