@@ -3,7 +3,8 @@ implementation in float64 on the device: width 6,144, 48 query and 8 key/value h
 feed-forward width 21,504, the 128,256-entry vocabulary, a window of 8,192 keys on the first
 layer, pages of 256 tokens.  A request of about 9,000 tokens runs in portions of 4,096 and
 then 40 single tokens, beside a short second request, in pools so small that the window
-group's pages are given back and used again (they are overwritten with NaN in between)."""
+group's pages are given back and used again (they are overwritten with NaN in between).  Once with
+every step launched kernel by kernel and once with the steps of a single token replayed from a graph."""
 
 import numpy as np
 import pytest
@@ -24,8 +25,9 @@ CONFIG = {
 PAGE = 256
 
 
+@pytest.mark.parametrize("graphs", [0, 2])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_two_layers_of_the_32b_width(dtype):
+def test_two_layers_of_the_32b_width(dtype, graphs):
     from cwm_amd.cache import CacheManager, CacheStorage
     from cwm_amd.engine import ModelRunner, Portion, random_model
     from cwm_amd.weights.random_init import random_tensor
@@ -47,7 +49,7 @@ def test_two_layers_of_the_32b_width(dtype):
     storage = CacheStorage(manager, device, model.runtime.act_dtype)
     for t in storage.paged.values():
         t.fill_(float("nan"))  # nothing is read that was not written
-    runner = ModelRunner(model, manager, storage)
+    runner = ModelRunner(model, manager, storage, num_graphs=graphs)  # with graphs, the steps of one token alone are replayed
     freed_pages = []
 
     def poison(group, gone):
@@ -83,6 +85,7 @@ def test_two_layers_of_the_32b_width(dtype):
             got[rid][pos] = logits[row].clone()
         cur += n
     assert short_cur == len(short_toks)
+    assert (runner.n_replays >= 30) == (graphs > 0), runner.n_replays
     # the window group gave pages back while the long request ran, and took them again
     window_group = next(g.index for g in manager.groups if g.window == 8192)
     assert any(g == window_group for g, _ in freed_pages)
