@@ -384,6 +384,29 @@ def test_sampling(vocab):
     assert int(toks[4]) == plain.greedy(logits[4])  # a vanishing nucleus keeps the top token
 
 
+@pytest.mark.parametrize("top_p", [1.0, 0.8])
+@pytest.mark.parametrize("vocab", [70, 1000, 5003, 128256])
+def test_sampling_draws_follow_the_inverse_cdf(vocab, top_p):
+    """512 uniform numbers over [0, 1), 0 and the largest float below 1 among them, on one row of logits:
+    every token has mass, the mass before it is at most u and the mass through it more than u (the search
+    goes through regions, parts and groups of 64 entries, and every edge between them is crossed here)."""
+    from cwm_amd import ops
+
+    g = torch.Generator().manual_seed(vocab + 1)
+    n = 512
+    logits = torch.randn(vocab, generator=g) * 2.0
+    us = torch.cat([torch.tensor([0.0, 1.0 - 2.0 ** -24]), torch.rand(n - 2, generator=g)])
+    toks, _, slp = ops.sample(logits.repeat(n, 1).to(DEV), torch.full((n,), 0.9).to(DEV), torch.full((n,), top_p).to(DEV), us.to(DEV))
+    toks, slp = toks.cpu().long(), slp.cpu()
+    probs = plain.sampling_probabilities(logits, 0.9, top_p).double()
+    c = torch.cumsum(probs, -1)
+    assert (probs[toks] > 0).all()
+    before = c[toks] - probs[toks]
+    assert (before <= us.double() + 1e-5).all() and (c[toks] >= us.double() - 1e-5).all()
+    torch.testing.assert_close(slp.double(), probs[toks].log(), rtol=1e-3, atol=1e-3)
+    assert len(set(toks.tolist())) > min(int((probs > 0).sum()), n) // 8  # the draws spread over the entries with mass
+
+
 def test_sampling_frequencies():
     """Draws with many uniform numbers follow the distribution (chi-square)."""
     from cwm_amd import ops
