@@ -128,7 +128,14 @@ class ModelRunner:
 
         plans = ops.StaticPlans(self.device, max_keys=table_width * page)
         batch = self._static_batch(portions, descriptor, table_width, plans, tokens_device)
-        logits = self.model.forward(batch, self.storage)  # this step; the work lists find their homes in it
+        try:
+            logits = self.model.forward(batch, self.storage)  # this step; the work lists find their homes in it
+        except ops.KernelError as exc:
+            # a kernel has no form of a fixed length for this model's steps: they are launched as they come (what
+            # the refused run has written to the cache, this run writes again)
+            print(f"[cwm_amd] decode steps are not captured as graphs: {exc}", file=sys.stderr, flush=True)
+            self.num_graphs = 0
+            return self.model.forward(build_batch(portions, self.manager, self.device, self.model.vocab_size, tokens_device), self.storage)
         try:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, pool=self._graph_pool):

@@ -117,3 +117,23 @@ def test_generation_with_and_without_graphs(folders, dtype, monkeypatch):
     for sampling in (False, True):
         for label in ("two", "none", "switch"):
             assert results[label, sampling] == results["default", sampling], f"{label}, sampling {sampling}"
+
+
+def test_a_model_whose_steps_have_no_fixed_form_is_launched_step_by_step(capfd):
+    """144 query heads on one key/value head: a decoded token's rows fill more than eight tiles, which go to
+    the kernel for blocks of many rows, and that has no work list of a fixed length.  The runner says so once
+    and launches every step; the logits are those of a run that never tried."""
+    from cwm_amd.replay import Replayer
+
+    config = {"architecture": "llama3_dense", "dim": 64, "n_layers": 2, "n_heads": 144, "n_kv_heads": 1, "head_dim": 16,
+              "vocab_size": 300, "hidden_dim": 96, "norm_eps": 1e-5, "rope_theta": 10000.0, "max_seq_len": 512}
+    requests = {"a": traces.random_tokens(1, 90, 300), "b": traces.random_tokens(2, 70, 300)}
+    steps = decode_steps(requests, tail=30)
+    outputs = {}
+    for graphs in (0, 2):
+        rep = Replayer(None, "bfloat16", traces.max_live_tokens(steps), page_size=16, random_config=config, seed=3, num_graphs=graphs)
+        outputs[graphs] = traces.run_in_process(rep, steps)
+        assert rep.runner.n_captures == 0 and rep.runner.n_replays == 0
+    assert "not captured as graphs" in capfd.readouterr().err
+    for step, want in outputs[0].items():
+        assert np.array_equal(outputs[2][step], want)
