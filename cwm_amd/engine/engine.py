@@ -29,7 +29,7 @@ from ..sampling.sampler import RequestStream, Sampler, effective_temperature
 from .api import GenArgs, Packet
 from .loading import load_model, random_model
 from .metrics import MetricsLog
-from .runner import ModelRunner
+from .runner import ModelRunner, weak_callback
 from .scheduler import Request, Scheduler
 
 
@@ -148,7 +148,7 @@ class Engine:
         self.scheduler = Scheduler(self.manager, args.max_batch, args.max_prefill, headroom=min(128, args.cache_block))
         self.sampler = Sampler(self.device)
         self.metrics = MetricsLog()
-        self.scheduler.on_event = self._scheduler_event
+        self.scheduler.on_event = weak_callback(self._scheduler_event)
         self._last_active = 0
         # a window of traced steps (cwm/fastgen/generate.py:148-156,397-434)
         self._profile_state = "inactive"

@@ -10,7 +10,9 @@ them in one call (cwm/fastgen/generate.py:480-498).
 
 from __future__ import annotations
 
+import gc
 import sys
+import weakref
 from collections import OrderedDict
 from dataclasses import dataclass
 from typing import Any, Callable, Hashable, List, Optional, Sequence
@@ -35,6 +37,19 @@ class CapturedStep:
     plans: Any  # ops.StaticPlans: the kernels' work lists, likewise
     tokens: torch.Tensor  # the descriptor's token ids
     logits: torch.Tensor  # where a replay leaves its logits
+
+
+def weak_callback(method: Callable) -> Callable:
+    """`method` (bound) as a callback that does not keep its object alive: an engine that registers its own
+    method with a part of itself would otherwise sit in a cycle of references, and its cache and graphs would
+    stay on the device until the collector finds it."""
+    ref = weakref.WeakMethod(method)
+
+    def call(*args: Any) -> Any:
+        target = ref()
+        return target(*args) if target is not None else None
+
+    return call
 
 
 class ModelRunner:
@@ -136,6 +151,12 @@ class ModelRunner:
             print(f"[cwm_amd] decode steps are not captured as graphs: {exc}", file=sys.stderr, flush=True)
             self.num_graphs = 0
             return self.model.forward(build_batch(portions, self.manager, self.device, self.model.vocab_size, tokens_device), self.storage)
+        # No graph may be destroyed while a stream captures (HIP refuses it, and an error in a destructor ends the
+        # process): whatever garbage holds one, a dropped engine for instance, is collected now, and the collector
+        # stays off until the capture has ended.
+        gc.collect()
+        collector_was_on = gc.isenabled()
+        gc.disable()
         try:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, pool=self._graph_pool):
@@ -145,6 +166,9 @@ class ModelRunner:
             self.num_graphs = 0
             self._captured.clear()
             return logits
+        finally:
+            if collector_was_on:
+                gc.enable()
         if self._graph_pool is None:
             self._graph_pool = graph.pool()
         self._captured[n] = CapturedStep(graph, descriptor, table_width, plans, batch.tokens, static_logits)

@@ -72,6 +72,7 @@ class Replayer:
     ) -> None:
         from .cache import CacheManager, CacheStorage
         from .engine import ModelRunner, load_model, random_model
+        from .engine.runner import weak_callback
 
         if max_tokens <= 0:
             raise ValueError("--max-tokens must be positive")
@@ -104,7 +105,7 @@ class Replayer:
         self._given: Dict[int, List[int]] = {}
         self._log = open(page_log, "w", encoding="utf-8") if page_log else None
         self._steps = 0
-        self.runner.on_pages_freed = self._pages_freed
+        self.runner.on_pages_freed = weak_callback(self._pages_freed)
 
     def _pages_freed(self, group: int, pages: List[int]) -> None:
         self._given.setdefault(group, []).extend(pages)

@@ -313,3 +313,25 @@ def test_decode_bursts_give_the_same_tokens_as_single_steps(tmp_path, monkeypatc
     tight, bursts_tight, _ = run(10, max_seq=96)
     for rid in prompts:
         assert tight[rid].tokens == single[rid].tokens
+
+
+def test_a_dropped_engine_is_freed_at_once(tmp_path, monkeypatch):
+    """An engine registers callbacks with its own scheduler; they must not keep it in a cycle of references,
+    or its cache (and its graphs) would stay on the device until the collector finds them, and a graph must
+    not be destroyed while another is captured."""
+    import gc
+    import weakref
+
+    folder = models.make_folder(tmp_path, "tiny_a", seed=2, dtype="float32")
+    gc.collect()
+    gc.disable()
+    try:
+        engine = _engine(folder, monkeypatch)
+        engine.generate_tokens([[1, 2, 3]], max_gen=3)
+        assert any(e.startswith("finish") for e in engine.scheduler.events)  # the callback is alive while the engine is
+        gone = weakref.ref(engine)
+        cache = weakref.ref(next(iter(engine.storage.paged.values())))
+        del engine
+        assert gone() is None and cache() is None
+    finally:
+        gc.enable()

@@ -137,3 +137,30 @@ def test_a_model_whose_steps_have_no_fixed_form_is_launched_step_by_step(capfd):
     assert "not captured as graphs" in capfd.readouterr().err
     for step, want in outputs[0].items():
         assert np.array_equal(outputs[2][step], want)
+
+
+def test_garbage_that_holds_a_graph_does_not_disturb_a_capture(folders):
+    """An engine with captured steps that only the collector can free (it sits in a cycle), and a collector set
+    to run at every opportunity: the next engine's capture collects first and keeps the collector off meanwhile
+    (destroying a graph while a stream captures is refused by HIP), and generates what it should."""
+    import gc
+
+    from cwm_amd.engine import Engine, GenArgs
+
+    vocab = configs.get("tiny_a")["vocab_size"]
+    prompts = [traces.random_tokens(5 + i, n, vocab) for i, n in enumerate([7, 20])]
+    args = GenArgs(use_sampling=False, max_batch=2, max_seq=1024, cache_block=8, max_prefill=64, sync_freq=4)
+    first = Engine.from_folder(folders["tiny_a", "bfloat16"], args, dtype="bfloat16")
+    want = first.generate_tokens(prompts, max_gen=30)
+    assert first.runner.n_captures > 0
+    cycle = [first]
+    cycle.append(cycle)
+    del first, cycle
+    thresholds = gc.get_threshold()
+    gc.set_threshold(1, 1, 1)
+    try:
+        second = Engine.from_folder(folders["tiny_a", "bfloat16"], args, dtype="bfloat16")
+        assert second.generate_tokens(prompts, max_gen=30) == want
+        assert second.runner.n_captures > 0
+    finally:
+        gc.set_threshold(*thresholds)
