@@ -68,10 +68,13 @@ LLAMA3_8B = {
     "max_seq_len": 8192,
 }
 LLAMA3_70B = dict(LLAMA3_8B, dim=8192, n_layers=80, n_heads=64, multiple_of=4096)
+# a small model of the same family (heads of 64): launching its kernels takes the host longer than running them takes the GPU
+SMALL_1B = dict(LLAMA3_8B, dim=2048, n_layers=16, n_heads=32, head_dim=64, ffn_dim_multiplier=1.5, multiple_of=256, max_seq_len=131072)
 SHAPES = {
     "cwm32b": ("CWM-32B shape (Llama-3 dense, 3 local : 1 global)", CWM_32B),
     "llama8b": ("Llama-3 8B shape (all layers global)", LLAMA3_8B),
     "llama70b": ("Llama-3 70B shape (all layers global)", LLAMA3_70B),
+    "small1b": ("16 layers of width 2,048 (32 heads of 64, all layers global)", SMALL_1B),
 }
 
 
