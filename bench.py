@@ -266,7 +266,7 @@ def main() -> int:
             if cache_bytes(args.batch, ctx) > 0.9 * free_bytes:  # an all-global shape at 131,072 tokens does not fit beside its weights
                 print(f"[bench] no point at context {ctx}: its cache does not fit", file=sys.stderr, flush=True)
                 continue
-            points[f"decode_b{args.batch}_ctx{ctx}"] = round(decode_run(args.batch, ctx, 10, 2)[0], 1)
+            points[f"decode_b{args.batch}_ctx{ctx}"] = round(decode_run(args.batch, ctx, 10, 6)[0], 1)  # (a capture, if any, falls into the warm-up)
         for b in (1, 8, 64):
             tok_s_b, median_ms, n_steps = engine_point(model, b, 1024, 256, page, typed.vocab_size)
             bytes_b = weight_bytes + cache_bytes(b, 1024 + 128)  # the context grows from 1,024 to 1,280 over the run

@@ -382,13 +382,17 @@ class Engine:
         for k in range(steps):
             portions = first if k == 0 else [Portion(rid=r.rid, tokens=[0], want=[0]) for r in requests]
             logits = self.runner.step(portions, tokens_device)
-            tokens_device, logprob, sample_logprob = self.sampler.sample_on_device(logits, params[0], params[1], params[2 + k])
-            results.append((tokens_device, logprob, sample_logprob))
+            packed = self.sampler.sample_packed(logits, params[0], params[1], params[2 + k])
+            tokens_device = packed[0]
+            results.append(packed)
         self.n_steps += steps
-        packed = torch.stack([torch.stack([t.to(torch.float64), a.to(torch.float64), b.to(torch.float64)]) for t, a, b in results]).cpu()
-        tokens = [[int(x) for x in packed[k, 0].tolist()] for k in range(steps)]
-        logprobs = [packed[k, 1].tolist() for k in range(steps)]
-        sample_logprobs = [packed[k, 2].tolist() for k in range(steps)]
+        host = torch.stack(results).cpu()  # [steps, 3, requests]: one copy for the whole burst
+        tokens, logprobs, sample_logprobs = [], [], []
+        for k in range(steps):
+            t, a, b = self.sampler.unpack(host[k])
+            tokens.append(t)
+            logprobs.append(a)
+            sample_logprobs.append(b)
         before = sum(len(r.generated) for r in requests)
         self.scheduler.burst_done(batch, tokens, self.stop_tokens, logprobs, sample_logprobs)
         self.n_generated += sum(len(r.generated) for r in requests) - before

@@ -998,15 +998,17 @@ def paged_attention(
 
 
 # --------------------------------------------------------------------------- #
-def sample(
+def sample_packed(
     logits: torch.Tensor,
     temperature: torch.Tensor,
     top_p: torch.Tensor,
     uniform: torch.Tensor,
-) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+) -> torch.Tensor:
     """Per row of float32 `logits` [R, V]: greedy where temperature <= 0, else a draw
     from softmax(logits / T) cut to the nucleus `top_p`, using the row's uniform
-    number.  Returns (tokens int32, logprobs, sample_logprobs)."""
+    number.  Returns one int32 tensor [3, R], so that everything reaches the host in one
+    copy: the tokens, then the bits of the float32 log-probabilities log softmax(logits)
+    at the token and of the token under the sampling distribution (`unpack_sampled`)."""
     _need_gpu(logits, temperature, top_p, uniform)
     if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
         raise KernelError("logits must be float32 [R, V] with contiguous rows")
@@ -1015,9 +1017,7 @@ def sample(
         if t.dtype != torch.float32 or t.numel() != n_rows or not t.is_contiguous():
             raise KernelError(f"{name} must be float32 [{n_rows}]")
     dev = logits.device
-    tokens = torch.empty(n_rows, dtype=torch.int32, device=dev)
-    logprob = torch.empty(n_rows, dtype=torch.float32, device=dev)
-    sample_logprob = torch.empty(n_rows, dtype=torch.float32, device=dev)
+    out = torch.empty((3, n_rows), dtype=torch.int32, device=dev)
     workspace = torch.empty((max(n_rows, 1), vocab), dtype=torch.float32, device=dev)
     lib = _build.load("sampling")
     _check(
@@ -1025,10 +1025,26 @@ def sample(
         lib.cwm_sample(
             _ptr(logits), ctypes.c_long(logits.stride(0) if n_rows > 1 else vocab), ctypes.c_int(n_rows),
             ctypes.c_int(vocab), _ptr(temperature), _ptr(top_p), _ptr(uniform), _ptr(workspace),
-            _ptr(tokens), _ptr(logprob), _ptr(sample_logprob), _stream(),
+            _ptr(out[0]), _ptr(out[1]), _ptr(out[2]), _stream(),
         ),
     )
-    return tokens, logprob, sample_logprob
+    return out
+
+
+def unpack_sampled(packed: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(tokens int32, logprobs float32, sample_logprobs float32) as views of what `sample_packed` returned
+    ([3, R], on any device)."""
+    return packed[0], packed[1].view(torch.float32), packed[2].view(torch.float32)
+
+
+def sample(
+    logits: torch.Tensor,
+    temperature: torch.Tensor,
+    top_p: torch.Tensor,
+    uniform: torch.Tensor,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """`sample_packed` as three tensors: (tokens int32, logprobs, sample_logprobs)."""
+    return unpack_sampled(sample_packed(logits, temperature, top_p, uniform))
 
 
 def token_logprobs(logits: torch.Tensor, rows: torch.Tensor, targets: torch.Tensor) -> torch.Tensor:
@@ -1072,5 +1088,7 @@ __all__ = [
     "mfma_attention_takes",
     "paged_attention",
     "sample",
+    "sample_packed",
+    "unpack_sampled",
     "token_logprobs",
 ]

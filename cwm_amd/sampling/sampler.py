@@ -50,6 +50,16 @@ class Sampler:
         the next step as they are."""
         return ops.sample(logits, temperatures, top_ps, uniforms)
 
+    def sample_packed(self, logits: torch.Tensor, temperatures: torch.Tensor, top_ps: torch.Tensor, uniforms: torch.Tensor) -> torch.Tensor:
+        """The same as one int32 tensor [3, R] (tokens, then the bits of the two log-probabilities), which
+        goes to the host in one copy; `unpack` reads it there."""
+        return ops.sample_packed(logits, temperatures, top_ps, uniforms)
+
+    @staticmethod
+    def unpack(packed: torch.Tensor) -> Tuple[List[int], List[float], List[float]]:
+        tokens, logprob, sample_logprob = ops.unpack_sampled(packed.cpu())
+        return tokens.tolist(), logprob.tolist(), sample_logprob.tolist()
+
     def sample(
         self,
         logits: torch.Tensor,
@@ -63,10 +73,4 @@ class Sampler:
         if not (len(temperatures) == len(top_ps) == len(uniforms) == n):
             raise ValueError("one temperature, top_p and uniform number per row of logits")
         params = torch.tensor([list(temperatures), list(top_ps), list(uniforms)], dtype=torch.float32).to(self.device)
-        tokens, logprob, sample_logprob = ops.sample(logits, params[0].contiguous(), params[1].contiguous(), params[2].contiguous())
-        packed = torch.stack([tokens.to(torch.float64), logprob.to(torch.float64), sample_logprob.to(torch.float64)]).cpu()
-        return (
-            [int(t) for t in packed[0].tolist()],
-            [float(x) for x in packed[1].tolist()],
-            [float(x) for x in packed[2].tolist()],
-        )
+        return self.unpack(ops.sample_packed(logits, params[0], params[1], params[2]))

@@ -163,6 +163,11 @@ def sample(logits, temperature, top_p, uniform):
     return toks, lp, slp
 
 
+def sample_packed(logits, temperature, top_p, uniform):
+    toks, lp, slp = sample(logits, temperature, top_p, uniform)
+    return torch.stack([toks, lp.float().view(torch.int32), slp.float().view(torch.int32)])
+
+
 def token_logprobs(logits, rows, targets):
     lp = torch.log_softmax(logits.float()[rows.long()], -1)
     return lp.gather(1, targets.long()[:, None])[:, 0]
@@ -174,6 +179,6 @@ def install(monkeypatch) -> None:
 
     for name in (
         "embedding", "add_rmsnorm", "silu_mul", "gate_up_silu", "linear", "gemm_f32", "gemm_bf16",
-        "rope_kv_write", "qkv_rope_write", "paged_attention", "sample", "token_logprobs",
+        "rope_kv_write", "qkv_rope_write", "paged_attention", "sample", "sample_packed", "token_logprobs",
     ):
         monkeypatch.setattr(ops, name, globals()[name])
