@@ -1,7 +1,7 @@
-"""One layer of the Llama-3 8B and of the 70B width through the step function, against the plain
-implementation in float64 on the device: widths 4,096 and 8,192 (the latter is longer than the products
-that keep a whole row of activations in registers take in one piece), 32 and 64 query heads on 8
-key/value heads of 128, feed-forward widths 14,336 and 28,672, pages of 256 tokens.  Two requests: one
+"""One layer of the Llama-3 8B and of the 70B width, and of a small one with heads of 64, through the step
+function, against the plain implementation in float64 on the device: widths 4,096, 8,192 (longer than the
+products that keep a whole row of activations in registers take in one piece) and 2,048; 32, 64 and 32 query
+heads on 8 key/value heads; feed-forward widths 14,336, 28,672 and 8,192; pages of 256 tokens.  Two requests: one
 prompt in portions of 300, 129 and 71 tokens, the other whole; then 24 steps of single tokens for both."""
 
 import pytest
@@ -13,14 +13,15 @@ from plain import llama3_plain
 pytestmark = pytest.mark.gpu
 
 WIDTHS = {
-    "8b": dict(dim=4096, n_heads=32, ffn_dim_multiplier=1.3, multiple_of=1024, hidden=14336),
-    "70b": dict(dim=8192, n_heads=64, ffn_dim_multiplier=1.3, multiple_of=4096, hidden=28672),
+    "8b": dict(dim=4096, n_heads=32, head_dim=128, ffn_dim_multiplier=1.3, multiple_of=1024, hidden=14336),
+    "70b": dict(dim=8192, n_heads=64, head_dim=128, ffn_dim_multiplier=1.3, multiple_of=4096, hidden=28672),
+    "small": dict(dim=2048, n_heads=32, head_dim=64, ffn_dim_multiplier=1.5, multiple_of=256, hidden=8192),
 }
 PAGE = 256
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("width", ["8b", "70b"])
+@pytest.mark.parametrize("width", ["8b", "70b", "small"])
 def test_one_layer_of_another_width(width, dtype):
     from cwm_amd.cache import CacheManager, CacheStorage
     from cwm_amd.engine import ModelRunner, Portion, random_model
@@ -28,7 +29,7 @@ def test_one_layer_of_another_width(width, dtype):
 
     w = WIDTHS[width]
     config = {
-        "architecture": "llama3_dense", "dim": w["dim"], "n_layers": 1, "n_heads": w["n_heads"], "n_kv_heads": 8, "head_dim": 128,
+        "architecture": "llama3_dense", "dim": w["dim"], "n_layers": 1, "n_heads": w["n_heads"], "n_kv_heads": 8, "head_dim": w["head_dim"],
         "vocab_size": 2048, "ffn_dim_multiplier": w["ffn_dim_multiplier"], "multiple_of": w["multiple_of"], "norm_eps": 1e-5,
         "pos_embed_impl": "rope", "rope_theta": 500000.0, "max_seq_len": 8192,
     }
