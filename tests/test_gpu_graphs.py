@@ -164,3 +164,25 @@ def test_garbage_that_holds_a_graph_does_not_disturb_a_capture(folders):
         assert second.runner.n_captures > 0
     finally:
         gc.set_threshold(*thresholds)
+
+
+def test_replays_across_the_step_from_few_to_many_partial_results(folders):
+    """A sequence that grows from 16,330 to 16,450 keys beside a short one: its chunks of 512 keys become more
+    than 32, from where another launch of the merge kernel takes its partial results; the capture was made with
+    room for that, and every replayed step gives the bits of the launched one."""
+    from cwm_amd.replay import Replayer
+
+    name, dtype = "tiny_a", "bfloat16"
+    vocab = configs.get(name)["vocab_size"]
+    requests = {"long": traces.random_tokens(3, 16450, vocab), "short": traces.random_tokens(4, 200, vocab)}
+    steps = decode_steps(requests, tail=120)
+    steps[0]["entries"] = [dict(e, want=[len(e["tokens"]) - 1]) for e in steps[0]["entries"]]
+    outputs = {}
+    for graphs in (0, 2):
+        rep = Replayer(folders[name, dtype], dtype, traces.max_live_tokens(steps), page_size=64, num_graphs=graphs)
+        outputs[graphs] = traces.run_in_process(rep, steps)
+        if graphs:
+            assert rep.runner.n_replays >= 110 and rep.runner.n_captures <= 4, (rep.runner.n_replays, rep.runner.n_captures)
+    for step, want in outputs[0].items():
+        assert np.isfinite(want).all()
+        assert np.array_equal(outputs[2][step], want), f"step {step} differs between the replayed and the launched run"
