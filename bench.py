@@ -306,6 +306,7 @@ def main() -> int:
             "points_prompt_tokens": 1024,
             "points_new_tokens": 256,
             "prefill_tokens": n_prefill,
+            "graphs": args.graphs,
         },
         "prefill": prefill,
         "roofline": {
