@@ -487,3 +487,123 @@ def test_toy_model_with_tied_head_scaled_embedding_and_two_kinds_of_norm():
         eps2 = eps2_saved
     finally:
         del ARCHITECTURES["toy_tied_model"]
+
+
+def test_toy_norm_and_toy_block_arrangement_register_build_and_step():
+    """A norm and an arrangement of a layer that the framework does not have, defined here: a norm that
+    centres each row before it scales it (with a weight and a bias), and a block in which mixer and
+    feed-forward both read the same normalised input and their results are added to the stream together.
+    Two such layers around the framework's own attention and feed-forward, float32, in portions and single
+    tokens against the whole-sequence computation below."""
+    from cwm_amd import ops
+    from cwm_amd.config import ARCHITECTURES, parse_config, register_architecture
+    from cwm_amd.models import Model
+    from cwm_amd.parts import Block, LayerCall, LayerPlan, ModelPlan, Norm, PartChoice, Runtime, TensorSpec, register_part
+    from cwm_amd.weights import random_tensors
+
+    class CentredNorm(Norm):
+        def __init__(self, dim, eps):
+            self.dim, self.eps = dim, eps
+
+        def tensor_specs(self):
+            return {"weight": TensorSpec((self.dim,), init="norm", precision="stored"), "bias": TensorSpec((self.dim,), precision="stored")}
+
+        def bind(self, tensors, runtime):
+            super().bind(tensors, runtime)
+            self.weight, self.bias = tensors["weight"].float(), tensors["bias"].float()
+
+        def forward(self, h, delta, rows=None):
+            total = h if delta is None else h + (delta.sum(0) if delta.dim() == 3 else delta).float()
+            if rows is None and delta is not None:
+                h.copy_(total)  # the residual sum, in place, in float32
+            x = total if rows is None else total[rows.long()]
+            x = x - x.mean(-1, keepdim=True)
+            x = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + self.eps)
+            return (x * self.weight + self.bias).to(self.runtime.act_dtype)
+
+    class ParallelBlock(Block):
+        """h += mixer(norm(h)) + feed_forward(norm(h)): one norm, two readers."""
+
+        def __init__(self, norm1, mixer, norm2, feed_forward, names):
+            self.norm, self.mixer, self.feed_forward, self.names = norm1, mixer, feed_forward, dict(names)
+
+        def _parts(self):
+            return {"norm1": self.norm, "mixer": self.mixer, "feed_forward": self.feed_forward}
+
+        def tensor_specs(self):
+            return {self.names[role] + n: s for role, part in self._parts().items() for n, s in part.tensor_specs().items()}
+
+        def bind(self, tensors, runtime):
+            super().bind(tensors, runtime)
+            for role, part in self._parts().items():
+                prefix = self.names[role]
+                part.bind({n[len(prefix):]: t for n, t in tensors.items() if n.startswith(prefix)}, runtime)
+
+        def forward(self, h, delta, batch, cache, write_cache=True):
+            x = self.norm.forward(h, delta)
+            a = self.mixer.forward(x, batch, cache, write_cache)
+            b = self.feed_forward.forward(x, batch)
+            dense = lambda t: (ops.sum_partials(t, torch.float32) if t.dim() == 3 else t.float())
+            return dense(a) + dense(b)
+
+    register_part("norm", "toy_centred", CentredNorm)
+    register_part("block", "toy_parallel", ParallelBlock)
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        architecture: str
+        dim: int
+        vocab_size: int
+
+    n_heads, n_kv, hd, theta, eps, hidden = 3, 1, 16, 300.0, 1e-3, 56
+
+    def toy_plan(cfg):
+        rope = PartChoice("rotary", {"head_dim": hd, "theta": theta})
+        norm = PartChoice("toy_centred", {"dim": cfg.dim, "eps": eps})
+        names = {"norm1": "ln.", "mixer": "attn.", "norm2": "unused.", "feed_forward": "ff."}
+        layers = [
+            LayerPlan(f"l{i}.", "toy_parallel", norm,
+                      PartChoice("paged_attention", {"dim": cfg.dim, "n_heads": n_heads, "n_kv_heads": n_kv, "head_dim": hd, "scale": hd**-0.5,
+                                                     "position_encoding": rope}),
+                      PartChoice("swiglu", {"dim": cfg.dim, "hidden_dim": hidden}), names)
+            for i in range(2)
+        ]
+        return ModelPlan(cfg.vocab_size, cfg.dim, "emb", layers, [LayerCall(0), LayerCall(1)], norm, "final", "head")
+
+    register_architecture("toy_parallel_model", ToyConfig, toy_plan)
+    try:
+        arch, cfg = parse_config({"architecture": "toy_parallel_model", "dim": 40, "vocab_size": 71})
+        model = Model(arch.build_plan(cfg))
+        assert not model.replayable  # the toy parts do not say that their steps may be captured: every step is launched
+        specs = model.tensor_specs()
+        assert "l1.ln.bias" in specs and not any(n.startswith("l0.unused.") for n in specs)
+        runtime = Runtime(torch.device("cuda:0"), torch.float32)
+        host = random_tensors(specs, seed=12, std=0.3, norm_init="uniform", dtype=torch.float32)
+        model.bind({k: v.to("cuda:0") for k, v in host.items()}, runtime)
+
+        def centred(x, w, b):
+            x = x - x.mean(-1, keepdim=True)
+            return x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * w + b
+
+        def whole_sequence(tokens):
+            w = {k: v.double() for k, v in host.items()}
+            n = len(tokens)
+            pos = torch.arange(n)
+            freqs = plain.rope_frequencies(hd, theta)
+            h = w["emb.weight"][torch.tensor(tokens)]
+            for i in range(2):
+                p = f"l{i}."
+                x = centred(h, w[p + "ln.weight"], w[p + "ln.bias"])
+                q = plain.rope_apply(plain.linear(x, w[p + "attn.wq.weight"]).view(n, n_heads, hd), pos, freqs)
+                k = plain.rope_apply(plain.linear(x, w[p + "attn.wk.weight"]).view(n, n_kv, hd), pos, freqs)
+                v = plain.linear(x, w[p + "attn.wv.weight"]).view(n, n_kv, hd)
+                a = plain.linear(plain.attention(q, k, v, scale=hd**-0.5).reshape(n, -1), w[p + "attn.wo.weight"])
+                h = h + a + plain.swiglu(x, w[p + "ff.w1.weight"], w[p + "ff.w2.weight"], w[p + "ff.w3.weight"])
+            return plain.linear(centred(h, w["final.weight"], w["final.bias"]), w["head.weight"]).float()
+
+        toks = {"a": traces.random_tokens(5, 23, 71), "b": traces.random_tokens(6, 9, 71)}
+        cut = _step_through(model, runtime, toks, [{"a": 5, "b": 2}, {"a": 1, "b": 1}, {"a": 1, "b": 6}, {"a": 16}])
+        for k in toks:
+            torch.testing.assert_close(cut[k], whole_sequence(toks[k]), rtol=2e-4, atol=2e-4)
+    finally:
+        del ARCHITECTURES["toy_parallel_model"]
