@@ -186,3 +186,75 @@ def test_replays_across_the_step_from_few_to_many_partial_results(folders):
     for step, want in outputs[0].items():
         assert np.isfinite(want).all()
         assert np.array_equal(outputs[2][step], want), f"step {step} differs between the replayed and the launched run"
+
+
+@pytest.mark.parametrize("says_so", [True, False])
+def test_a_part_from_outside_opts_into_captured_steps(says_so):
+    """An attention defined here that normalises query and key heads between projection and rotation
+    (`transform_qk`): decode steps of its model are captured only if it says that the hook keeps to the rule
+    of captured steps (`transform_replayable`), and then give the bits of launched steps."""
+    from dataclasses import dataclass
+
+    from cwm_amd.cache import CacheManager, CacheStorage
+    from cwm_amd.config import ARCHITECTURES, parse_config, register_architecture
+    from cwm_amd.engine import ModelRunner, Portion
+    from cwm_amd.models import Model
+    from cwm_amd.parts import LayerCall, LayerPlan, ModelPlan, PartChoice, Runtime, register_part
+    from cwm_amd.parts.attention import PagedAttention
+    from cwm_amd.parts.base import MIXERS
+    from cwm_amd.weights import random_tensors
+
+    class UnitNormAttention(PagedAttention):
+        transform_replayable = says_so
+
+        def transform_qk(self, q, k, batch):
+            for t in (q, k):
+                if t is not None:
+                    t.copy_(torch.nn.functional.normalize(t.float(), dim=-1).to(t.dtype))
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        architecture: str
+        dim: int
+        vocab_size: int
+
+    def toy_plan(cfg):
+        rope = PartChoice("rotary", {"head_dim": 16, "theta": 100.0})
+        attn = PartChoice("toy_unit_norm_attention_for_graphs", {"dim": cfg.dim, "n_heads": 4, "n_kv_heads": 2, "head_dim": 16, "scale": 3.0,
+                                                                 "position_encoding": rope})
+        names = {"norm1": "n1.", "mixer": "attn.", "norm2": "n2.", "feed_forward": "ff."}
+        norm = PartChoice("rmsnorm", {"dim": cfg.dim, "eps": 1e-5})
+        layer = LayerPlan("l0.", "pre_norm", norm, attn, PartChoice("swiglu", {"dim": cfg.dim, "hidden_dim": 48}), names)
+        return ModelPlan(cfg.vocab_size, cfg.dim, "emb", [layer], [LayerCall(0)], norm, "final", "head")
+
+    register_part("mixer", "toy_unit_norm_attention_for_graphs", UnitNormAttention)
+    register_architecture("toy_graph_model", ToyConfig, toy_plan)
+    try:
+        arch, cfg = parse_config({"architecture": "toy_graph_model", "dim": 32, "vocab_size": 83})
+        model = Model(arch.build_plan(cfg))
+        runtime = Runtime(torch.device("cuda:0"), torch.bfloat16)
+        host = random_tensors(model.tensor_specs(), seed=2, std=0.2, norm_init="uniform", dtype=torch.bfloat16)
+        model.bind({k: v.to("cuda:0") for k, v in host.items()}, runtime)
+        assert model.replayable == says_so
+        toks = {"a": traces.random_tokens(1, 70, 83), "b": traces.random_tokens(2, 45, 83)}
+        outputs = {}
+        for graphs in (0, 2):
+            manager = CacheManager(model.cache_specs, 8, 32, 2)
+            storage = CacheStorage(manager, runtime.device, runtime.act_dtype)
+            runner = ModelRunner(model, manager, storage, num_graphs=graphs)
+            out = []
+            for rid in toks:
+                runner.admit(rid)
+                assert manager.extend(rid, 5)
+                runner.step([Portion(rid, toks[rid][:5], [])])
+            for i in range(5, 45):
+                for rid in toks:
+                    assert manager.extend(rid, 1)
+                out.append(runner.step([Portion(rid, [toks[rid][i]], [0]) for rid in toks]).cpu())
+            outputs[graphs] = torch.stack(out)
+            if graphs:
+                assert (runner.n_replays > 30) == says_so and (runner.n_captures > 0) == says_so
+        assert torch.isfinite(outputs[0]).all() and torch.equal(outputs[0], outputs[2])
+    finally:
+        del ARCHITECTURES["toy_graph_model"]
+        del MIXERS["toy_unit_norm_attention_for_graphs"]
