@@ -5,7 +5,9 @@
 
 Default run: the layer sizes of the CWM-32B shape with random weights, a batch of 8
 requests at a context of 32,768 tokens each; a step is one decode step of the whole
-batch through the engine's step function and sampler.  It prints one JSON line:
+batch through the engine's step function and sampler, each step fed on the device by the
+tokens that the one before sampled, with a host round trip every ten steps (the engine's
+`sync_freq`, the reference's way of decoding).  It prints one JSON line:
 `value` is decoded tokens a second; `prefill` is a 2,048-token prompt in one step;
 `roofline` compares the bytes a decode step has to read (every weight once, and the
 cache of the live requests) with the HBM peak.  The cache of the timed requests is filled
@@ -192,24 +194,28 @@ def main() -> int:
                 assert manager.extend(b, n)
                 manager.advance(b, n)
                 held += n
-        tokens = [(17 * b + 3) % vocab for b in range(batch)]
-        temps, top_ps, us = [0.0] * batch, [1.0] * batch, [0.0] * batch
+        # as the engine decodes (sync_freq, cwm/fastgen/generate.py:729-809): every step's tokens are sampled on the
+        # device and feed the next step from there; they come to the host once in ten steps
+        tokens = torch.tensor([(17 * b + 3) % vocab for b in range(batch)], dtype=torch.int32, device=device)
+        params = torch.zeros((3, batch), dtype=torch.float32, device=device)
+        params[1] = 1.0  # temperature 0 (greedy), top-p 1, uniform numbers 0
+        placeholder = [Portion(b, [0], [0]) for b in range(batch)]  # the token ids come from the device
 
-        def one_step(tokens):
-            portions = []
-            for b in range(batch):
-                assert manager.extend(b, 1)
-                portions.append(Portion(b, [tokens[b]], [0]))
-            logits = runner.step(portions)
-            new, _, _ = sampler.sample(logits, temps, top_ps, us)
-            return new
+        def run(n_steps, tokens):
+            for i in range(n_steps):
+                for b in range(batch):
+                    assert manager.extend(b, 1)
+                logits = runner.step(placeholder, tokens_device=tokens)
+                packed = sampler.sample_packed(logits, params[0], params[1], params[2])
+                tokens = packed[0]
+                if i % 10 == 9:
+                    packed.cpu()
+            return tokens
 
-        for _ in range(warmup):
-            tokens = one_step(tokens)
+        tokens = run(warmup, tokens)
         torch.cuda.synchronize()
         start = time.perf_counter()
-        for _ in range(steps):
-            tokens = one_step(tokens)
+        tokens = run(steps, tokens)
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - start
         del runner, manager
