@@ -407,6 +407,23 @@ def test_sampling_draws_follow_the_inverse_cdf(vocab, top_p):
     assert len(set(toks.tolist())) > min(int((probs > 0).sum()), n) // 8  # the draws spread over the entries with mass
 
 
+def test_sampling_keeps_all_entries_equal_to_the_nucleus_threshold():
+    """Where entries are exactly equal at the nucleus' edge the reference's sort keeps some of them, whichever
+    come first (cwm/fastgen/utils/sampling.py:38-45); the kernel keeps all of them, so that the draw does not
+    depend on an order among equals.  Two equal largest logits and a vanishing nucleus: both are kept, each with
+    probability one half, and the uniform number picks between them in vocabulary order."""
+    from cwm_amd import ops
+
+    vocab = 1000
+    logits = torch.randn(vocab, generator=torch.Generator().manual_seed(3))
+    logits[[17, 640]] = 9.0
+    us = torch.tensor([0.0, 0.49, 0.51, 0.99])
+    n = us.numel()
+    toks, _, slp = ops.sample(logits.repeat(n, 1).to(DEV), torch.full((n,), 0.7).to(DEV), torch.full((n,), 1e-6).to(DEV), us.to(DEV))
+    assert toks.cpu().tolist() == [17, 17, 640, 640]
+    torch.testing.assert_close(slp.cpu(), torch.full((n,), math.log(0.5)), rtol=1e-5, atol=1e-5)
+
+
 def test_sampling_frequencies():
     """Draws with many uniform numbers follow the distribution (chi-square)."""
     from cwm_amd import ops
