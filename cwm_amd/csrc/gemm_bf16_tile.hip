@@ -5,7 +5,8 @@
 // no longer fits a block's registers.
 //
 // Persistent blocks of eight wavefronts.  A block computes a tile of C: a block of 64 or 128 rows by
-// up to TL_GROUPS groups of 16 columns, in steps of TL_BK = 64 along K.  The step's pieces of W
+// up to TL_GROUPS groups of 16 columns (above 128 rows: sixteen wavefronts, 256 rows by up to
+// TL_TALL_GROUPS groups), in steps of TL_BK = 64 along K.  The step's pieces of W
 // [columns][64 k] and of A [rows][64 k] reach LDS by direct loads (global_load_lds_dwordx4: lane l
 // of a wavefront fills bytes 16 l .. 16 l + 15 after a uniform address), two or three steps ahead
 // into three or four buffers, so a step costs no registers, no LDS writes and one barrier.  A row
@@ -28,7 +29,7 @@
 //     block that is the s-th to touch a tile writes its float32 partial sum into slab s,
 //     C[s][M][N], and the block that ends a tile zeroes the slabs it leaves unused, so the consumer
 //     adds `slabs` slabs whatever the cut (as it adds the streaming kernel's partial sums).
-// Cut and order of every sum are fixed by N, K, the block height (64 rows, or multiples of 128) and
+// Cut and order of every sum are fixed by N, K, the block height (64, 128 or 256 rows) and
 // the number of blocks; within one block height a row's result does not depend on the other rows.
 //
 // Replaces torch.nn.functional.linear at cwm/fastgen/forward.py:593-606,763,776-782,820 for such
@@ -54,6 +55,11 @@ extern "C" int cwm_gemm_bf16_tile_max_rows() { return TL_MAX_ROWS; }
 #ifndef TL_WAVES_128
 #define TL_WAVES_128 8  // and of a block of 128 rows
 #endif
+// More than 128 rows: blocks of 256 rows and 16 wavefronts, so that W is still read once; its tiles are at most
+// TL_TALL_GROUPS wide (three buffers of 256 rows and 128 columns fill the LDS)
+#define TL_TALL_ROWS 256
+#define TL_TALL_WAVES 16
+#define TL_TALL_GROUPS 8
 
 // G: groups of 16 columns that a step's piece of W holds (the widest tile of the cut)
 template <int BM, int WAVES, int G, typename TC, bool GLU>
@@ -72,6 +78,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restric
   constexpr int W_DMA = W_BYTES / 1024 / WAVES;  // loads of a wavefront per step: each fills 1 KB = 8 rows
   constexpr int A_DMA = A_BYTES / 1024 / WAVES;
   static_assert(G % WN == 0 && BM % (16 * WM) == 0 && W_BYTES % (1024 * WAVES) == 0 && A_BYTES % (1024 * WAVES) == 0, "block shape");
+  static_assert(TL_SHARED_GROUPS <= TL_TALL_GROUPS && STAGES * STAGE <= 160 * 1024, "a block's buffers must fit the LDS");
   __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * STAGE];
 
   const int tid = threadIdx.x;
@@ -272,7 +279,8 @@ static int most_sharers(long tiles, long steps, long chunk) {
 
 static TilePlan tile_plan(int M, int N, int K, int units) {
   TilePlan p;
-  p.block_rows = M <= 64 ? 64 : 128;
+  p.block_rows = M <= 64 ? 64 : M <= 128 ? 128 : TL_TALL_ROWS;
+  const int widest_whole = p.block_rows == TL_TALL_ROWS ? TL_TALL_GROUPS : TL_GROUPS;
   p.n_row_blocks = (M + p.block_rows - 1) / p.block_rows;
   p.n_groups = N / 16;
   p.steps = K / TL_BK;
@@ -283,7 +291,7 @@ static TilePlan tile_plan(int M, int N, int K, int units) {
     const long col_tiles = tiles / p.n_row_blocks;
     if (col_tiles > p.n_groups) break;
     const long widest = (p.n_groups + col_tiles - 1) / col_tiles;
-    if (widest > TL_GROUPS) continue;
+    if (widest > widest_whole) continue;
     if (p.n_groups / col_tiles < TL_MIN_GROUPS) break;
     p.n_col_tiles = (int)col_tiles;
     p.total = tiles * p.steps;
@@ -337,21 +345,23 @@ extern "C" int cwm_gemm_bf16_tile(const void* A, long lda, const void* W, long l
   hipLaunchKernelGGL((gemm_tile_kernel<BM, WAVES, G, TC, GLU>), grid, dim3(WAVES * 64), 0, stream, (const bf16_t*)A, lda, \
                      (const bf16_t*)W, ldw, (TC*)C, ldc, slab_stride, M, N, p.steps, p.n_groups, p.n_col_tiles,           \
                      p.n_row_blocks, p.total, p.chunk, p.slabs)
-#define CWM_LAUNCH_ROWS(BM, WAVES)                             \
+#define CWM_LAUNCH_ROWS(BM, WAVES, WHOLE)                       \
   do {                                                         \
     if (glu)                                                   \
-      CWM_LAUNCH_TILE(BM, WAVES, TL_GROUPS, bf16_t, true);     \
+      CWM_LAUNCH_TILE(BM, WAVES, WHOLE, bf16_t, true);         \
     else if (slabs > 1)                                        \
       CWM_LAUNCH_TILE(BM, WAVES, TL_SHARED_GROUPS, float, false); \
     else if (c_dtype == CWM_F32)                               \
-      CWM_LAUNCH_TILE(BM, WAVES, TL_GROUPS, float, false);     \
+      CWM_LAUNCH_TILE(BM, WAVES, WHOLE, float, false);         \
     else                                                       \
-      CWM_LAUNCH_TILE(BM, WAVES, TL_GROUPS, bf16_t, false);    \
+      CWM_LAUNCH_TILE(BM, WAVES, WHOLE, bf16_t, false);        \
   } while (0)
   if (p.block_rows == 64)
-    CWM_LAUNCH_ROWS(64, TL_WAVES_64);
+    CWM_LAUNCH_ROWS(64, TL_WAVES_64, TL_GROUPS);
+  else if (p.block_rows == 128)
+    CWM_LAUNCH_ROWS(128, TL_WAVES_128, TL_GROUPS);
   else
-    CWM_LAUNCH_ROWS(128, TL_WAVES_128);
+    CWM_LAUNCH_ROWS(TL_TALL_ROWS, TL_TALL_WAVES, TL_TALL_GROUPS);
 #undef CWM_LAUNCH_ROWS
 #undef CWM_LAUNCH_TILE
   return cwm_launch_status("gemm_bf16_tile");

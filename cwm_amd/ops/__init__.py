@@ -555,7 +555,7 @@ def gemm_bf16_tile(
     units: Optional[int] = None,
 ) -> torch.Tensor:
     """bfloat16 x [M <= 512, K] @ weight[N, K]^T with float32 sums: persistent blocks whose tiles
-    of 64 or 128 rows reach LDS by direct loads and that share the work by steps of K.  Returns
+    of 64, 128 or 256 rows reach LDS by direct loads and that share the work by steps of K.  Returns
     [M, N]; with `partials_ok` it may return float32 partial sums [P, M, N] for the caller to add.
     `glu`: the weight's rows are gate and up rows in alternating groups of 8 and the result is
     silu(gate) * up, [M, N / 2] (in the kernel where a block owns whole tiles, else after it).
@@ -613,8 +613,9 @@ def gemm_bf16_tile(
 # batch 16: 15.3 against 15.6 ms)
 STREAM_FUSED_ROWS = 8
 STREAM_EPILOGUE_ROWS = 16
-TILE_ROWS = 128  # rows up to which the tiled product reads W once
-TILE_ROWS_SHARED = 256  # rows up to which it still beats the library where blocks share tiles (a narrow result)
+TILE_ROWS = 128  # rows up to which the tiled product is the fastest whatever the shape
+TILE_TALL_ROWS = 256  # rows of its tallest block: up to there it reads W once
+TILE_COLUMNS = 128  # columns of a tall block's tile
 
 
 def _prefers_tile(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> bool:
@@ -623,20 +624,20 @@ def _prefers_tile(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Te
 
 
 def _tile_wins(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    """Whether the tiled product takes this product and is the fastest for it (measured on the 32B
-    shape's matrices: above 128 rows W is read once per 128 rows, which the library beats on wide results)."""
+    """Whether the tiled product takes this product and is the fastest for it.  Above 128 rows its blocks of
+    256 rows are bound by LDS and matrix cores, and the library is faster wherever its own tiles fill the
+    chip.  Measured on the matrices of the 8B, 32B and 70B shapes at 160 and 256 rows: the tiled product,
+    which shares K between blocks, is ahead where its tiles are at most half as many as the compute units
+    (up to 16,384 columns: 41 against 67 us for the 32B shape's q/k/v product at 256 rows, 89 against 234 us
+    for its feed-forward's second product).  With two blocks of rows (up to 512) it was ahead on that second
+    product alone (144 against 195 us at 384 rows), which the float32 partial sums that the next kernel then
+    reads cost again in a decode step, so more than 256 rows go to the library."""
     m = x.shape[0]
-    if m > TILE_ROWS_SHARED or not _tile_takes(x, weight):
+    if m > TILE_TALL_ROWS or not _tile_takes(x, weight):
         return False
     if m <= TILE_ROWS:
         return True
-    lib = _build.load("gemm_bf16_tile")
-    units = _compute_units(x.device)
-    key = (m, weight.shape[0], x.shape[1], units)
-    slabs = _tile_slabs.get(key)
-    if slabs is None:
-        slabs = _tile_slabs[key] = int(lib.cwm_gemm_bf16_tile_slabs(*key))
-    return slabs > 1
+    return 2 * -(-weight.shape[0] // TILE_COLUMNS) <= _compute_units(x.device)
 
 
 def _stream_takes(x: torch.Tensor, weight: torch.Tensor) -> bool:
@@ -660,7 +661,7 @@ def gemm_bf16(
     """bfloat16 x [M, K] @ bfloat16 weight[N, K]^T, float32 accumulation.
 
     Up to 8 rows: the hand-written persistent weight-streaming kernel, x in registers.
-    Up to 128 rows (256 for a narrow result): the hand-written tiled kernel, x and W
+    Up to 128 rows (256 for a result of at most 16,384 columns): the hand-written tiled kernel, x and W
     through LDS (it needs K % 64 == 0 and N % 16 == 0; other sizes of up to 64 rows stream).
     More rows: the library product (hipBLASLt through torch), as the reference calls a
     library here, with a bfloat16 or a float32 result.  Row lengths that are no multiple

@@ -71,7 +71,7 @@ def test_two_layers_of_the_32b_width(dtype, graphs):
             runner.admit("short")
         if k >= 5 and short_cur < len(short_toks):
             # its prompt in portions beside the long request's decoded tokens: steps of 131, 101 and 71 rows, which
-            # the products take in blocks of 128 rows twice, once, and in a block of 64
+            # the products take in a block of 256 rows (or the library), of 128 and of 64
             m = min([130, 100, 70][min(k - 5, 2)], len(short_toks) - short_cur)
             assert manager.extend("short", m)
             swant = sorted({0, m // 2, m - 1})
