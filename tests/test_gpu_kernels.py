@@ -1059,3 +1059,58 @@ def test_gemm_bf16_tile_random_sizes(seed):
             got = ops.gemm_bf16_tile(a.to(DEV), w.to(DEV), None, torch.bfloat16, glu=True, units=units)
             two = ops.silu_mul(ops.gemm_bf16_tile(a.to(DEV), w.to(DEV), None, torch.bfloat16, units=units), grouped=True)
             assert torch.equal(got, two), (m, n, k, units)
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd", [(16, 8, 64), (48, 8, 128), (6, 3, 48)])
+def test_attention_of_a_decoded_token_does_not_depend_on_the_batch(n_q, n_kv, hd):
+    """Decoded tokens of 200 sequences in one call (another shape of block and another way of reading the work
+    items than a few sequences get) and the same sequences ten at a time: the same bits, and what float32 torch
+    gives."""
+    from types import SimpleNamespace
+
+    from cwm_amd import ops
+
+    page_size, n_seqs = 16, 200
+    g = torch.Generator().manual_seed(n_q + hd)
+    lens = [int(x) for x in torch.randint(70, 1400, (n_seqs,), generator=g)]
+    lens[3], lens[7] = 2049, 4100  # other chunk lengths
+    scale = hd ** -0.5
+    pages_of = [(n + page_size - 1) // page_size for n in lens]
+    total_pages = sum(pages_of) + 1
+    perm = torch.randperm(total_pages, generator=g)
+    width = max(pages_of)
+    table = torch.full((n_seqs, width), -1, dtype=torch.int32)
+    cache = torch.full((total_pages, 2, n_kv, page_size * hd), float("nan"), dtype=torch.bfloat16)
+    kc = cache[:, 0].view(total_pages, n_kv, page_size, hd)
+    vc = cache[:, 1].view(total_pages, n_kv, page_size // 8, hd, 8)
+    q = torch.randn((n_seqs, n_q, hd), generator=g).to(torch.bfloat16)
+    want, used = [], 0
+    for b, n in enumerate(lens):
+        k = torch.randn((n, n_kv, hd), generator=g).to(torch.bfloat16)
+        v = torch.randn((n, n_kv, hd), generator=g).to(torch.bfloat16)
+        table[b, : pages_of[b]] = perm[used : used + pages_of[b]].to(torch.int32)
+        used += pages_of[b]
+        pos = torch.arange(n)
+        pages, slots = table[b, pos // page_size].long(), pos % page_size
+        kc[pages, :, slots, :] = k
+        vc[pages, :, slots // 8, :, slots % 8] = v
+        if b % 20 == 0:
+            group = n_q // n_kv
+            scores = torch.einsum("hd,khd->hk", q[b].float(), k.float().repeat_interleave(group, dim=1)) * scale
+            want.append((b, torch.einsum("hk,khd->hd", torch.softmax(scores, -1), v.float().repeat_interleave(group, dim=1)).reshape(-1)))
+    cache_d, table_d = cache.to(DEV), table.to(DEV)
+
+    def run(which):
+        batch = SimpleNamespace(
+            q_lens=[1] * len(which), kv_lens=[lens[b] for b in which], n_seqs=len(which), n_tokens=len(which), scratch={},
+            cu_q=torch.arange(len(which) + 1, dtype=torch.int32).to(DEV), kv_len=torch.tensor([lens[b] for b in which], dtype=torch.int32).to(DEV),
+        )
+        rows = torch.tensor(which)
+        return ops.paged_attention_mfma(q[rows].to(DEV), cache_d, table_d[rows.to(DEV)].contiguous(), batch, None, scale).cpu()
+
+    together = run(list(range(n_seqs)))
+    assert torch.isfinite(together).all()
+    for start in range(0, n_seqs, 10):
+        assert torch.equal(run(list(range(start, start + 10))), together[start : start + 10]), f"sequences {start}.. differ"
+    for b, w in want:
+        torch.testing.assert_close(together[b].float(), w, rtol=2e-2, atol=2e-2)
