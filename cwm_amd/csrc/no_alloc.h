@@ -13,6 +13,11 @@
 // left in it.  Calls that overlap on one GPU (two streams, two threads) race on it:
 // the caller must order them.  Nothing in the array has to start at zero: every
 // element a call reads it has written before.
+//
+// The array's address on a GPU is looked up at the first call on that GPU
+// (hipGetSymbolAddress, under a mutex), which is not a call for a stream that is
+// capturing: call `cwm_sample_static_init` (or `cwm_sample_static` once) on each device
+// before any capture; later calls only launch kernels.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -30,6 +35,10 @@ extern "C" int cwm_sample_static(const float* logits, long row_stride, int n_row
                                  const float* temperature, const float* top_p, const float* uniform,
                                  int* token_out, float* logprob_out, float* sample_logprob_out,
                                  hipStream_t stream);
+
+// Looks up the array's address on the current device (once; later calls return at once).  Allocates
+// nothing.  Returns non-zero with a message if the address cannot be found.
+extern "C" int cwm_sample_static_init();
 
 // floats of the array (CWM_SAMPLE_STATIC_MAX_FLOATS), for callers that size their batches by it
 extern "C" long cwm_sample_static_capacity();

@@ -347,6 +347,29 @@ static std::mutex sample_scratch_mutex;
 
 extern "C" long cwm_sample_static_capacity() { return CWM_SAMPLE_STATIC_MAX_FLOATS; }
 
+// The array's address on the current device, looked up at the first call there.  Sets `*out`; returns non-zero on failure.
+static int sample_scratch_on_current_device(float** out) {
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess) return cwm_fail("sample_static: hipGetDevice failed: %s", hipGetErrorString(err));
+  CWM_REQUIRE(device >= 0 && device < CWM_MAX_DEVICES, "sample_static: device %d is outside 0..%d", device, CWM_MAX_DEVICES - 1);
+  std::lock_guard<std::mutex> guard(sample_scratch_mutex);
+  if (sample_scratch_ptr[device] == nullptr) {
+    void* found = nullptr;
+    err = hipGetSymbolAddress(&found, HIP_SYMBOL(sample_scratch));
+    if (err != hipSuccess || found == nullptr)
+      return cwm_fail("sample_static: the scratch array has no address on device %d: %s", device, hipGetErrorString(err));
+    sample_scratch_ptr[device] = (float*)found;
+  }
+  *out = sample_scratch_ptr[device];
+  return 0;
+}
+
+extern "C" int cwm_sample_static_init() {
+  float* scratch = nullptr;
+  return sample_scratch_on_current_device(&scratch);
+}
+
 extern "C" int cwm_sample_static(const float* logits, long row_stride, int n_rows, int vocab,
                                  const float* temperature, const float* top_p, const float* uniform,
                                  int* token_out, float* logprob_out, float* sample_logprob_out,
@@ -357,22 +380,8 @@ extern "C" int cwm_sample_static(const float* logits, long row_stride, int n_row
               "sample_static: %d rows of %d logits need %lld floats of scratch, the fixed array holds %d", n_rows, vocab,
               (long long)n_rows * vocab, CWM_SAMPLE_STATIC_MAX_FLOATS);
   if (n_rows == 0) return 0;
-  int device = -1;
-  hipError_t err = hipGetDevice(&device);
-  if (err != hipSuccess) return cwm_fail("sample_static: hipGetDevice failed: %s", hipGetErrorString(err));
-  CWM_REQUIRE(device >= 0 && device < CWM_MAX_DEVICES, "sample_static: device %d is outside 0..%d", device, CWM_MAX_DEVICES - 1);
   float* scratch = nullptr;
-  {
-    std::lock_guard<std::mutex> guard(sample_scratch_mutex);
-    if (sample_scratch_ptr[device] == nullptr) {
-      void* found = nullptr;
-      err = hipGetSymbolAddress(&found, HIP_SYMBOL(sample_scratch));
-      if (err != hipSuccess || found == nullptr)
-        return cwm_fail("sample_static: the scratch array has no address on device %d: %s", device, hipGetErrorString(err));
-      sample_scratch_ptr[device] = (float*)found;
-    }
-    scratch = sample_scratch_ptr[device];
-  }
+  if (int status = sample_scratch_on_current_device(&scratch)) return status;
   launch_sample(logits, row_stride, n_rows, vocab, temperature, top_p, uniform, scratch, token_out, logprob_out, sample_logprob_out, stream);
   return cwm_launch_status("sample_static");
 }

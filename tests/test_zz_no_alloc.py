@@ -32,16 +32,20 @@ def _outputs(rows, device):
     )
 
 
-def test_sample_static_equals_sample_on_two_calls_in_a_row():
+# a large call first, then a smaller one (fewer rows, a shorter vocabulary): once with vocabularies that are no
+# multiple of 4 (rows read entry by entry) and once with multiples of 4, as real vocabularies are (rows read 16
+# bytes at a time); rows 1, 3, ... have a nucleus of 0.8, so the second call of each pair has one too
+@pytest.mark.parametrize("calls", [[(7, 4099), (3, 1237)], [(5, 4096), (2, 1024)]])
+def test_sample_static_equals_sample_on_two_calls_in_a_row(calls):
     from cwm_amd.ops import build
 
     lib = build.load("sampling")
+    assert lib.cwm_sample_static_init() == 0, lib.cwm_error_message()
     lib.cwm_sample_static_capacity.restype = ctypes.c_long
     capacity = lib.cwm_sample_static_capacity()
     device = torch.device("cuda:0")
     stream = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
-    # a large call first, then a smaller one (fewer rows, a shorter vocabulary that is no power of two)
-    for seed, (rows, vocab) in enumerate([(7, 4099), (3, 1237)]):
+    for seed, (rows, vocab) in enumerate(calls):
         assert rows * vocab <= capacity
         logits, temperature, top_p, uniform = _inputs(seed, rows, vocab, device)
         want = _outputs(rows, device)
@@ -65,6 +69,22 @@ def test_sample_static_equals_sample_on_two_calls_in_a_row():
         # greedy rows are the argmax
         greedy = [r for r in range(rows) if float(temperature[r]) == 0.0]
         assert got[0][greedy].cpu().tolist() == logits[greedy].argmax(dim=1).cpu().tolist()
+        # the other rows against the distribution itself (softmax at the temperature, the nucleus of
+        # cwm/fastgen/utils/sampling.py:38-41, inverse CDF in the order of the vocabulary),
+        # so that a mistake shared by both entry points would show
+        for r in range(rows):
+            if r in greedy:
+                continue
+            probs = torch.softmax(logits[r].double().cpu() / float(temperature[r]), -1)
+            order = torch.argsort(probs, descending=True)
+            before = torch.cumsum(probs[order], 0) - probs[order]
+            keep = torch.zeros_like(probs, dtype=torch.bool)
+            keep[order[before <= float(top_p[r])]] = True  # an entry stays while the mass before it is within top_p
+            probs = torch.where(keep, probs, torch.zeros_like(probs))
+            probs = probs / probs.sum()
+            cdf = torch.cumsum(probs, 0)
+            tok, u = int(got[0][r]), float(uniform[r])
+            assert probs[tok] > 0 and float(cdf[tok] - probs[tok]) <= u + 1e-4 and float(cdf[tok]) >= u - 1e-4
 
 
 def test_sample_static_refuses_more_than_its_array_holds():
