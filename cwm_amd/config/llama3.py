@@ -115,6 +115,10 @@ class Llama3DenseConfig:
             raise ConfigError(f"dim {self.dim} is not a multiple of n_heads {self.n_heads} and head_dim is not given")
         if self.head_size % 2 != 0:
             raise ConfigError(f"head_dim {self.head_size} must be even for rotary pairs")
+        if self.attn_impl != "xformers":
+            # the one value the reference accepts (cwm/model/transformer.py:134); it names the reference's attention
+            # library, which this engine's own kernels stand in for, so any other value is a configuration of something else
+            raise ConfigError(f"attn_impl must be 'xformers' (cwm/model/transformer.py:134), found {self.attn_impl!r}")
         if self.weight_tying:
             raise ConfigError("weight_tying is not supported (cwm/model/transformer.py:135)")
         if self.q_lora_rank or self.kv_lora_rank:

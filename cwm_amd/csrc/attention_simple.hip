@@ -93,6 +93,14 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
   int seg_len;
   const int n_seg = segments_of(p - start + 1, seg_len);
   if (seg >= n_seg) return;
+  if (n_seg > (int)gridDim.y || (n_seg > 1 && partial == nullptr)) {
+    // the caller's `max_keys` was below what this token reads: the launch has no block (or no scratch) for
+    // some of its segments.  Its rows come out NaN; nothing else is touched.
+    if (seg == 0)
+      for (int e = threadIdx.x; e < nh * head_dim; e += SIMPLE_WAVES * CWM_WAVE)
+        Elem<T>::store(out + (size_t)t * out_stride + (size_t)h0 * head_dim + e, __uint_as_float(0x7fc00000u));
+    return;
+  }
   const int k0 = start + seg * seg_len;
   const int k1 = min(p + 1, k0 + seg_len);  // exclusive
 
@@ -335,7 +343,8 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
 template <typename T>
 __global__ void __launch_bounds__(CWM_WAVE)
 attention_simple_join_kernel(T* __restrict__ out, long out_stride, const float* __restrict__ partial,
-                             const int* __restrict__ positions, int n_q_heads, int head_dim, int window_left) {
+                             const int* __restrict__ positions, int n_q_heads, int head_dim, int window_left,
+                             int max_segments) {
   const int t = blockIdx.x / n_q_heads;
   const int h = blockIdx.x - t * n_q_heads;
   const int lane = threadIdx.x;
@@ -343,7 +352,7 @@ attention_simple_join_kernel(T* __restrict__ out, long out_stride, const float* 
   const int start = window_left >= 0 ? max(0, p - window_left) : 0;
   int seg_len;
   const int n_seg = segments_of(p - start + 1, seg_len);
-  if (n_seg <= 1) return;
+  if (n_seg <= 1 || n_seg > max_segments) return;  // more than the launch had room for: the rows are NaN already
   const float neg_inf = -__builtin_inff();
   const float* base = partial + (((size_t)t * n_q_heads + h) * SIMPLE_MAX_SEGMENTS) * PARTIAL_STRIDE(head_dim);
   float m_all = neg_inf;
@@ -373,7 +382,8 @@ attention_simple_join_kernel(T* __restrict__ out, long out_stride, const float* 
 
 // `max_keys`: the most keys that any token of the call reads (its position + 1, or the window if that
 // is less); `partial`: float32 scratch of n_tokens * n_q_heads * 16 * (head_dim + 2) values, needed
-// (and touched) only if max_keys exceeds 2,048.
+// (and touched) only if max_keys exceeds 2,048.  A token that reads more keys than `max_keys` says has no
+// place for its segments' results: its rows of `out` are NaN and every kernel ends normally.
 extern "C" int cwm_attention_simple(const void* q, long q_stride, void* out, long out_stride, const void* cache,
                                     int dtype, const int* block_table, int table_width, const int* positions,
                                     const int* seq_of_token, int n_tokens, int n_q_heads, int n_kv_heads,
@@ -428,7 +438,7 @@ extern "C" int cwm_attention_simple(const void* q, long q_stride, void* out, lon
 #undef CWM_LAUNCH_SIMPLE
     if (max_segments > 1)
       hipLaunchKernelGGL(attention_simple_join_kernel<float>, dim3((unsigned)join_blocks), dim3(CWM_WAVE), 0, stream,
-                         (float*)out, out_stride, (const float*)partial, positions, n_q_heads, head_dim, window_left);
+                         (float*)out, out_stride, (const float*)partial, positions, n_q_heads, head_dim, window_left, max_segments);
   } else if (dtype == CWM_BF16) {
     hipLaunchKernelGGL((attention_simple_kernel<bf16_t, SIMPLE_HEADS, SIMPLE_D_REGS>), grid, dim3(SIMPLE_WAVES * CWM_WAVE), 0, stream, (const bf16_t*)q,
                        q_stride, (bf16_t*)out, out_stride, (const bf16_t*)cache, block_table, table_width, positions,
@@ -436,7 +446,7 @@ extern "C" int cwm_attention_simple(const void* q, long q_stride, void* out, lon
                        scale);
     if (max_segments > 1)
       hipLaunchKernelGGL(attention_simple_join_kernel<bf16_t>, dim3((unsigned)join_blocks), dim3(CWM_WAVE), 0, stream,
-                         (bf16_t*)out, out_stride, (const float*)partial, positions, n_q_heads, head_dim, window_left);
+                         (bf16_t*)out, out_stride, (const float*)partial, positions, n_q_heads, head_dim, window_left, max_segments);
   } else {
     return cwm_fail("attention: unknown dtype %d", dtype);
   }

@@ -14,9 +14,12 @@ control back.
 
 from __future__ import annotations
 
+import logging
 import os
 import queue
+import signal
 import time
+import weakref
 from typing import Any, Dict, Generator, Hashable, Iterable, List, Optional, Sequence, Union
 
 import torch
@@ -245,6 +248,26 @@ class Engine:
             self.metrics.record("unpark", tokens=len(request))
         elif kind == "preempt":
             self.metrics.record("preempt", tokens=len(request))
+
+    def install_profile_signal(self, profile_sig: int = signal.SIGUSR2) -> bool:
+        """Make `profile_sig` (SIGUSR2, as the reference's default) call `request_profile`, so that a window
+        of steps can be traced from outside the process (`kill -USR2 PID`); cwm/fastgen/generate.py:139,
+        159-169,405-406.  As there, a handler that is already set is left alone (returns False).  Only the
+        main thread can set a handler.  The handler holds the engine weakly."""
+        log = logging.getLogger("cwm_amd")
+        if signal.getsignal(profile_sig) is not signal.SIG_DFL:
+            log.warning("Signal handler for %s is set; the profile handler was not installed", profile_sig)
+            return False
+        ref = weakref.ref(self)
+
+        def handler(_signum: int, _frame: Any) -> None:
+            engine = ref()
+            if engine is not None:
+                engine.request_profile()
+
+        signal.signal(profile_sig, handler)
+        log.info("Profiling signal handler set for signal %s", profile_sig)
+        return True
 
     def request_profile(self) -> None:
         """Trace the next `profile_iters` steps (FG_PROFILE_ITERS, default 8) with torch's

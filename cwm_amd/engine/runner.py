@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import gc
 import sys
+import threading
 import weakref
 from collections import OrderedDict
 from dataclasses import dataclass
@@ -37,6 +38,12 @@ class CapturedStep:
     plans: Any  # ops.StaticPlans: the kernels' work lists, likewise
     tokens: torch.Tensor  # the descriptor's token ids
     logits: torch.Tensor  # where a replay leaves its logits
+
+
+# HIP refuses the destruction of a graph while any stream of the process captures, and torch ends the process when
+# that happens in a destructor.  Every capture and every drop of a captured step in this module holds this lock, so
+# that runners on several threads do not destroy one runner's graphs during another's capture.
+_GRAPH_LOCK = threading.RLock()
 
 
 def weak_callback(method: Callable) -> Callable:
@@ -81,6 +88,23 @@ class ModelRunner:
         self._graph_pool: Any = None
         self.n_captures = 0
         self.n_replays = 0
+
+    def __del__(self) -> None:
+        # the captured steps' graphs go here, under the lock, not whenever the last reference happens to fall
+        captured = getattr(self, "_captured", None)
+        if captured:
+            with _GRAPH_LOCK:
+                captured.clear()
+
+    def _drop_capture(self, n: Optional[int] = None, oldest: bool = False) -> None:
+        """Destroy the capture of `n` requests, the least recently used one, or (neither given) all of them."""
+        with _GRAPH_LOCK:
+            if oldest:
+                self._captured.popitem(last=False)
+            elif n is None:
+                self._captured.clear()
+            else:
+                self._captured.pop(n, None)
 
     # ---- requests ------------------------------------------------------------- #
     def admit(self, rid: Hashable) -> int:
@@ -133,7 +157,11 @@ class ModelRunner:
                 self._captured.move_to_end(n)
                 self.n_replays += 1
                 return held.logits.clone()  # the next replay writes there again
-        self._captured.pop(n, None)  # outgrown: its tables or work lists have no room for this step
+        if held is not None:
+            # outgrown: its tables or work lists have no room for this step.  Whether a step of so many requests is
+            # still worth a capture at the lengths it has now is measured anew.
+            self._drop_capture(n)
+            self._host_share.pop(n, None)
         if self.graphs_where_host_bound and not self._worth_a_capture(n):
             return self._launched_and_timed(portions, tokens_device, n)
         table_width = width + max(width // 4, 2)
@@ -154,27 +182,36 @@ class ModelRunner:
         # No graph may be destroyed while a stream captures (HIP refuses it, and an error in a destructor ends the
         # process): whatever garbage holds one, a dropped engine for instance, is collected now, and the collector
         # stays off until the capture has ended.
-        gc.collect()
-        collector_was_on = gc.isenabled()
-        gc.disable()
-        try:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
-                static_logits = self.model.forward(batch, self.storage)
-        except Exception as exc:  # the step above has run and stands; later ones are launched kernel by kernel
-            print(f"[cwm_amd] decode steps are not captured as graphs: {type(exc).__name__}: {exc}", file=sys.stderr, flush=True)
-            self.num_graphs = 0
-            self._captured.clear()
-            return logits
-        finally:
-            if collector_was_on:
-                gc.enable()
-        if self._graph_pool is None:
-            self._graph_pool = graph.pool()
-        self._captured[n] = CapturedStep(graph, descriptor, table_width, plans, batch.tokens, static_logits)
-        self.n_captures += 1
-        while len(self._captured) > self.num_graphs:
-            self._captured.popitem(last=False)
+        # (The collector's switch is the process's: it covers this thread's garbage and, with the lock, other
+        # runners' captured steps; a graph that other code of the process destroys on another thread is not covered.)
+        with _GRAPH_LOCK:
+            gc.collect()
+            collector_was_on = gc.isenabled()
+            gc.disable()
+            try:
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, pool=self._graph_pool):
+                    static_logits = self.model.forward(batch, self.storage)
+            except Exception as exc:  # the step above has run and stands; later ones are launched kernel by kernel
+                print(f"[cwm_amd] decode steps are not captured as graphs: {type(exc).__name__}: {exc}", file=sys.stderr, flush=True)
+                self.num_graphs = 0
+                self._captured.clear()
+                self._graph_pool = None
+                # the stream must have left capture mode and the device must answer, or later launches would fail
+                # with an error that names none of this
+                if torch.cuda.is_current_stream_capturing():
+                    raise RuntimeError("a failed capture of a decode step left the stream capturing") from exc
+                torch.cuda.synchronize(self.device)
+                return logits
+            finally:
+                if collector_was_on:
+                    gc.enable()
+            if self._graph_pool is None:
+                self._graph_pool = graph.pool()
+            self._captured[n] = CapturedStep(graph, descriptor, table_width, plans, batch.tokens, static_logits)
+            self.n_captures += 1
+            while len(self._captured) > self.num_graphs:
+                self._drop_capture(oldest=True)
         return logits
 
     def _worth_a_capture(self, n: int) -> bool:

@@ -116,6 +116,7 @@ def main(argv: Optional[List[str]] = None) -> int:
         engine = Engine.from_random(config, args.weight_seed, args.gen_args, args.dtype, args.device, args.stop_tokens, args.seed)
     else:
         engine = Engine.from_folder(args.checkpoint_dir, args.gen_args, args.dtype, args.device, args.stop_tokens, args.seed)
+    engine.install_profile_signal()  # kill -USR2 PID traces a window of steps (FG_PROFILE_ITERS, FG_PROFILE_DIR)
     log.info("cache: %d tokens in pages of %d; max_batch %d", engine.max_seq, args.gen_args.cache_block, args.gen_args.max_batch)
 
     q: "queue.Queue[Optional[Packet]]" = queue.Queue()

@@ -80,11 +80,14 @@ class PagedAttention(Mixer):
         weights = {n: tensors[f"{n}.weight"] for n in names}
         biases = {n: tensors.get(f"{n}.bias") for n in names}
         pairing = self.position_encoding.rotary_pairing() if self.position_encoding is not None else "adjacent"
+        # element j of a head as `transform_qk` sees it is element qk_order[j] of the head as the folder's wq and wk give it
+        self.qk_order = torch.arange(self.head_dim)
         if pairing == "halves":
             # the kernels turn adjacent elements: bring element i and i + head_dim / 2 of every query and key
             # head side by side, once, by the order of the projections' rows
             half = self.head_dim // 2
             order = torch.stack([torch.arange(half), torch.arange(half) + half], dim=1).reshape(-1)
+            self.qk_order = order
             for n, heads in (("wq", self.n_heads), ("wk", self.n_kv_heads)):
                 rows = (torch.arange(heads)[:, None] * self.head_dim + order[None, :]).reshape(-1).to(weights[n].device)
                 weights[n] = weights[n][rows]
@@ -102,7 +105,13 @@ class PagedAttention(Mixer):
         `q` [T, Hq, hd] and keys `k` [T, Hkv, hd] (None when this call writes no cache) in place
         here (a norm per head, say) before they are rotated and the keys are cached.  Overriding it
         takes the step off the fused projection + rotation + cache-write kernel, and off captured
-        steps unless the subclass sets `transform_replayable`."""
+        steps unless the subclass sets `transform_replayable`.
+
+        The elements of a head arrive in the order the kernels rotate them, which for a position
+        encoding with the "halves" pairing is not the folder's: element j here is element
+        `self.qk_order[j]` of the head as wq and wk give it (`qk_order` is the identity for adjacent
+        pairs; it is set by `bind`).  A subclass with a tensor per element of a head (the weight of a
+        norm) reorders it once, `weight[self.qk_order]`, after calling `bind` of this class."""
 
     transform_replayable = False  # whether an overriding `transform_qk` keeps to the rule of `Part.replayable`
 

@@ -139,11 +139,48 @@ def gather(steps: List[dict], outputs: Dict[int, np.ndarray], lengths: Dict[str,
     return result
 
 
-def run_in_process(replayer, steps: List[dict]) -> Dict[int, np.ndarray]:
+class PageUse:
+    """Which (request, logical page) every physical page of every layer group has served, read off the
+    manager's block tables.  `note` is called whenever tables may have changed (after pages were taken:
+    right after `extend`, or after a step if nothing can both take and give back in between)."""
+
+    def __init__(self, manager) -> None:
+        self.manager = manager
+        self.served: Dict[int, Dict[int, set]] = {g.index: {} for g in manager.groups}
+
+    def note(self) -> None:
+        for g in self.manager.groups:
+            for rid in self.manager.live_requests():
+                for logical, page in enumerate(self.manager.table(g.index, rid)):
+                    if page >= 0:
+                        self.served[g.index].setdefault(page, set()).add((rid, logical))
+
+    def pages_used_again(self, group: int) -> int:
+        """Physical pages of the group that have held more than one (request, logical page)."""
+        return sum(1 for users in self.served[group].values() if len(users) > 1)
+
+    def pages_shared_between_requests(self, group: int) -> int:
+        return sum(1 for users in self.served[group].values() if len({rid for rid, _ in users}) > 1)
+
+
+def run_in_process(replayer, steps: List[dict], page_use: "PageUse | None" = None) -> Dict[int, np.ndarray]:
     outputs = {}
-    for st in steps:
-        out = replayer.step(st["entries"], st["end"])
-        if out is not None:
-            outputs[st["step"]] = out
-        replayer.manager.check()
+    if page_use is not None:
+        # the replayer takes a step's pages before it runs the step and gives pages back after it
+        inner = replayer.runner.step
+
+        def step_and_note(portions):
+            page_use.note()
+            return inner(portions)
+
+        replayer.runner.step = step_and_note
+    try:
+        for st in steps:
+            out = replayer.step(st["entries"], st["end"])
+            if out is not None:
+                outputs[st["step"]] = out
+            replayer.manager.check()
+    finally:
+        if page_use is not None:
+            del replayer.runner.step
     return outputs

@@ -46,6 +46,7 @@ def test_reference_layer_rule_and_big_shapes():
     ({"weight_tying": True}, "weight_tying"),
     ({"kv_lora_rank": 16}, "latent"),
     ({"qk_norm": True}, "qk_norm"),
+    ({"attn_impl": "sdpa"}, "attn_impl"),
     ({"pos_embed_impl": "alibi"}, "pos_embed_impl"),
     ({"scaled_rope": {"scale_factor": 1}}, "scale_factor"),
     ({"scaled_rope": {"low_freq_factor": 8, "high_freq_factor": 4}}, "wavelength"),

@@ -335,3 +335,35 @@ def test_a_dropped_engine_is_freed_at_once(tmp_path, monkeypatch):
         assert gone() is None and cache() is None
     finally:
         gc.enable()
+
+
+def test_profile_window_by_signal(tmp_path, monkeypatch):
+    """SIGUSR2 asks for a profile window from outside the process, as the reference's handler does
+    (cwm/fastgen/generate.py:159-169,405-406); a handler that someone else has set is left alone."""
+    import os
+    import signal
+
+    monkeypatch.setenv("FG_PROFILE_ITERS", "1")
+    monkeypatch.setenv("FG_PROFILE_DIR", str(tmp_path))
+    folder = models.make_folder(tmp_path, "tiny_a", seed=2, dtype="float32")
+    vocab = configs.get("tiny_a")["vocab_size"]
+    engine = _engine(folder, monkeypatch)
+    saved = signal.getsignal(signal.SIGUSR2)
+    try:
+        signal.signal(signal.SIGUSR2, signal.SIG_DFL)
+        assert engine.install_profile_signal() is True
+        assert engine._profile_state == "inactive"
+        os.kill(os.getpid(), signal.SIGUSR2)
+        for _ in range(100):  # the handler runs between bytecodes of the main thread
+            if engine._profile_state == "requested":
+                break
+        assert engine._profile_state == "requested"
+        engine.generate_tokens([traces.random_tokens(1, 9, vocab)], max_gen=3)
+        assert engine.last_profile_path is not None and os.path.exists(engine.last_profile_path)
+        # a second engine finds the first one's handler set and leaves it
+        assert _engine(folder, monkeypatch).install_profile_signal() is False
+        # the handler does not keep its engine alive, and outlives it harmlessly
+        del engine
+        os.kill(os.getpid(), signal.SIGUSR2)
+    finally:
+        signal.signal(signal.SIGUSR2, saved)

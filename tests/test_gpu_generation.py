@@ -108,6 +108,46 @@ def test_sampled_generation_equals_the_plain_draw(tmp_path):
         assert run([rid])[rid] == want[rid], f"{rid} alone"
 
 
+@pytest.mark.parametrize("name", ["tiny_b", "tiny_d"])
+@pytest.mark.parametrize("sampling", [False, True])
+def test_bfloat16_generation_through_the_engine_against_the_plain_logits(tmp_path, name, sampling):
+    """bfloat16 through the whole engine (scheduler, portions of 24 tokens, bursts of decode steps fed on the
+    device, decode steps replayed from graphs, six requests over four places so that they come and go): the
+    log-probabilities that the engine returns for the prompt's and for its own generated tokens are those of
+    the plain implementation on prompt + generated tokens, within what bfloat16 rounding costs there (a logit
+    error of e moves a log-probability by at most 2e), and every greedy token lies that near the top."""
+    import queue
+
+    from cwm_amd.engine import Engine, GenArgs, Packet
+
+    folder = models.make_folder(tmp_path, name, seed=8, dtype="bfloat16")
+    vocab = configs.get(name)["vocab_size"]
+    prompts = {i: traces.random_tokens(300 + i, n, vocab) for i, n in enumerate([5, 33, 64, 90, 12, 41])}
+    args = GenArgs(use_sampling=sampling, temperature=0.8, top_p=0.9, max_batch=4, max_seq=4096, cache_block=8, max_prefill=24,
+                   logprobs=True, prompt_logprobs=True, num_cuda_graphs=16, sync_freq=5)
+    engine = Engine.from_folder(folder, args, dtype="bfloat16")
+    q = queue.Queue()
+    for rid, prompt in prompts.items():
+        q.put(Packet(thread_id=rid, tokens=list(prompt), max_gen=40))
+    q.put(None)
+    packets = {pkt.thread_id: pkt for pkt in engine.generate(q) if pkt is not None}
+    assert engine.runner.n_replays > 0 and engine.n_steps > engine.n_iterations  # graphs and bursts were in it
+    for rid, prompt in prompts.items():
+        pkt = packets[rid]
+        toks = list(prompt) + list(pkt.tokens)
+        assert len(pkt.tokens) == 40 and len(pkt.logprobs) == len(toks) - 1
+        want = cmp.expected(folder, {"x": toks}, "bfloat16")["x"]
+        exact = torch.log_softmax(torch.from_numpy(want.exact).double(), -1)
+        limit = 2 * cmp.BF16_MAX_RATIO * want.max
+        for place in range(len(toks) - 1):  # the logits after token `place` score token `place + 1`
+            plain_lp = float(exact[place, toks[place + 1]])
+            assert abs(pkt.logprobs[place] - plain_lp) <= limit, (
+                f"{name} request {rid}: log-probability of token {place + 1} is {pkt.logprobs[place]:.5f}, plain {plain_lp:.5f}, limit {limit:.2e}")
+            if not sampling and place >= len(prompt) - 1:
+                row = want.exact[place]
+                assert row[toks[place + 1]] >= row.max() - limit, f"{name} request {rid}: generated token {place + 1 - len(prompt)} is not near the top"
+
+
 def test_a_request_without_max_gen_runs_until_the_cache_is_full(tmp_path):
     """max_gen None in the options and in the packet: the request's longest length is the cache's
     (cwm/fastgen/generate.py:91-96), and it ends with reason "length" there."""

@@ -354,6 +354,127 @@ def test_attention_far_key_stands_out():
     torch.testing.assert_close(out_w2[1], v[far, 0], rtol=1e-3, atol=1e-3)
 
 
+def _simple_segments(n_keys):
+    """The plain kernel's rule for cutting a token's keys (the comment at the head of
+    cwm_amd/csrc/attention_simple.hip): one segment up to 2,048 keys, then ceil(n / 1,024) segments, at most
+    16, of equal length in chunks of 64."""
+    n_seg = 1 if n_keys <= 2048 else min(16, -(-n_keys // 1024))
+    return n_seg, -(-(-(-n_keys // n_seg)) // 64) * 64
+
+
+def _loud_keys_case(lengths, page_size, seed):
+    """Sequences of the given lengths in a float32 cache (one key/value head of 64, eight query heads), pages
+    in reverse order.  For the last token of every sequence each query head has a key of its own that answers
+    it loudly: at position 0, at the last and the first key of adjacent segments, at the query's own position."""
+    n_q, hd = 8, 64
+    g = torch.Generator().manual_seed(seed)
+    pages_of = [(n + page_size - 1) // page_size for n in lengths]
+    table = torch.full((len(lengths), max(pages_of)), -1, dtype=torch.int32)
+    total = sum(pages_of)
+    cache = torch.full((total, 2, 1, page_size * hd), float("nan"))
+    kc = cache[:, 0].view(total, 1, page_size, hd)
+    vc = cache[:, 1].view(total, 1, page_size // 8, hd, 8)
+    used, seqs = 0, []
+    for b, n in enumerate(lengths):
+        n_seg, seg_len = _simple_segments(n)
+        if n_seg > 1:
+            loud = [0, seg_len - 1, seg_len, (n_seg - 1) * seg_len - 1, (n_seg - 1) * seg_len, n - 1, n // 2, seg_len // 2]
+        else:
+            loud = [0, 63, 64, 255, 256, n - 1, n // 2, n - 2]
+        assert len(set(loud)) == n_q and max(loud) < n
+        k = torch.randn((n, hd), generator=g) * 0.1
+        v = torch.randn((n, hd), generator=g)
+        q = torch.randn((n_q, hd), generator=g)
+        for h, j in enumerate(loud):
+            k[j] = q[h] * 40.0
+        table[b, :pages_of[b]] = torch.arange(total - used - 1, total - used - 1 - pages_of[b], -1, dtype=torch.int32)
+        used += pages_of[b]
+        pos = torch.arange(n)
+        pages, slots = table[b, pos // page_size].long(), pos % page_size
+        kc[pages, 0, slots, :] = k
+        vc[pages, 0, slots // 8, :, slots % 8] = v
+        seqs.append(dict(n=n, k=k, v=v, q=q, loud=loud))
+    return seqs, cache, table
+
+
+def _exact_last_row(s, window):
+    n, hd = s["n"], 64
+    scores = (s["q"].double() @ s["k"].double().T) * hd ** -0.5  # [heads, keys]
+    if window is not None:
+        scores[:, : max(0, n - window)] = float("-inf")
+    return torch.softmax(scores, -1) @ s["v"].double()
+
+
+def test_attention_simple_segments_and_their_edges():
+    """The plain kernel's segmented path in float32: one launch with tokens of 1, 3, 5 and 16 segments (600,
+    2,049, 5,000 and 17,000 keys; the last is held at the cap of 16), `max_keys` given.  Every query head has
+    its own loud key: the first key, the last key of a segment and the first of the next, the query's own.  A
+    key dropped or counted twice at an edge changes that head's output by the whole of a value."""
+    from cwm_amd import ops
+
+    lengths, page_size, hd = [600, 2049, 5000, 17000], 16, 64
+    assert [_simple_segments(n)[0] for n in lengths] == [1, 3, 5, 16]
+    seqs, cache, table = _loud_keys_case(lengths, page_size, seed=21)
+    q = torch.stack([s["q"] for s in seqs]).to(DEV)
+    positions = torch.tensor([n - 1 for n in lengths], dtype=torch.int32).to(DEV)
+    seq = torch.arange(len(lengths), dtype=torch.int32).to(DEV)
+    cache_d, table_d = cache.to(DEV), table.to(DEV)
+    out = ops.paged_attention_simple(q, cache_d, table_d, positions, seq, None, hd ** -0.5, max_keys=max(lengths)).cpu().view(len(lengths), 8, hd)
+    for b, s in enumerate(seqs):
+        torch.testing.assert_close(out[b].double(), _exact_last_row(s, None), rtol=1e-4, atol=1e-4)
+        for h, j in enumerate(s["loud"]):
+            torch.testing.assert_close(out[b, h], s["v"][j], rtol=1e-3, atol=1e-3)
+    # the same rows one sequence at a time, `max_keys` from the positions: bit-equal (the cut depends on the token alone)
+    for b in range(len(lengths)):
+        alone = ops.paged_attention_simple(q[b:b + 1], cache_d, table_d, positions[b:b + 1], seq[b:b + 1], None, hd ** -0.5).cpu().view(8, hd)
+        assert torch.equal(alone, out[b])
+
+
+@pytest.mark.parametrize("n,far", [(5000, 100), (17000, 0), (17000, 613), (2700, 7)])
+def test_attention_simple_window_edge_on_the_segmented_path(n, far):
+    """A window whose first key is the loud one sees it; one key shorter does not; both windows hold more than
+    2,048 keys, so the window's first key is a segment's first key."""
+    from cwm_amd import ops
+
+    page_size, hd = 8, 64
+    seqs, cache, table = _loud_keys_case([n], page_size, seed=n + far)
+    s = seqs[0]
+    s["k"][far] = s["q"][3] * 40.0  # head 3 has a second loud key, at `far`; its own lies at (n_seg-1)*seg_len-1
+    own = s["loud"][3]
+    page, slot = int(table[0, far // page_size]), far % page_size
+    cache[page, 0].view(1, page_size, hd)[0, slot] = s["k"][far]
+    positions = torch.tensor([n - 1], dtype=torch.int32).to(DEV)
+    seq = torch.zeros(1, dtype=torch.int32).to(DEV)
+    for window, sees in ((n - far, True), (n - far - 1, False)):
+        assert _simple_segments(window)[0] > 1
+        out = ops.paged_attention_simple(s["q"][None].to(DEV), cache.to(DEV), table.to(DEV), positions, seq, window, hd ** -0.5, max_keys=n).cpu().view(8, hd)
+        torch.testing.assert_close(out.double(), _exact_last_row(s, window), rtol=1e-4, atol=1e-4)
+        both = (s["v"][far] + s["v"][own]) / 2  # two keys equally loud share the row
+        if sees:
+            torch.testing.assert_close(out[3], both, rtol=1e-3, atol=1e-3)
+        else:
+            torch.testing.assert_close(out[3], s["v"][own], rtol=1e-3, atol=1e-3)
+
+
+def test_attention_simple_with_too_small_max_keys_gives_nan_and_ends_normally():
+    """`max_keys` below what a token reads leaves no block or no scratch for its segments: its rows are NaN,
+    the other tokens' rows are right, and every kernel ends normally (the next call works)."""
+    from cwm_amd import ops
+
+    lengths, page_size, hd = [600, 5000], 16, 64
+    seqs, cache, table = _loud_keys_case(lengths, page_size, seed=4)
+    q = torch.stack([s["q"] for s in seqs]).to(DEV)
+    positions = torch.tensor([n - 1 for n in lengths], dtype=torch.int32).to(DEV)
+    seq = torch.arange(2, dtype=torch.int32).to(DEV)
+    cache_d, table_d = cache.to(DEV), table.to(DEV)
+    for max_keys in (1000, 3000):  # no scratch at all; scratch, but three segments where five are needed
+        out = ops.paged_attention_simple(q, cache_d, table_d, positions, seq, None, hd ** -0.5, max_keys=max_keys).cpu().view(2, 8, hd)
+        assert torch.isnan(out[1]).all()
+        torch.testing.assert_close(out[0].double(), _exact_last_row(seqs[0], None), rtol=1e-4, atol=1e-4)
+    out = ops.paged_attention_simple(q, cache_d, table_d, positions, seq, None, hd ** -0.5, max_keys=5000).cpu().view(2, 8, hd)
+    torch.testing.assert_close(out[1].double(), _exact_last_row(seqs[1], None), rtol=1e-4, atol=1e-4)
+
+
 @pytest.mark.parametrize("vocab", [263, 1000, 128256])
 def test_sampling(vocab):
     from cwm_amd import ops
@@ -550,6 +671,70 @@ def test_attention_mfma_long_ranges(window):
         cu_q=torch.tensor(cu, dtype=torch.int32).to(DEV), kv_len=torch.tensor(kv_lens, dtype=torch.int32).to(DEV),
     )
     got = ops.paged_attention_mfma(torch.cat(q_rows).to(DEV), cache.to(DEV), table.to(DEV), batch, window, scale).cpu()
+    assert torch.isfinite(got).all()
+    torch.testing.assert_close(got.float(), torch.cat(want_rows), rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("window", [None, 8192])
+def test_attention_mfma_long_ranges_with_heads_of_128_and_pages_of_256(window):
+    """The geometry of a long-context decode step of the 32B shape (48 query heads on 8 key/value heads
+    of 128, pages of 256 keys): decoded tokens after 32,767 and 131,071 keys (chunks of 512 and 1,024 keys,
+    up to 128 partial results a row) and a portion of three rows after 100,000, against float32 torch on
+    the device.  Everything is made on the device; one far key stands out for the longest sequence."""
+    from types import SimpleNamespace
+
+    from cwm_amd import ops
+
+    n_q, n_kv, hd, page_size = 48, 8, 128, 256
+    group = n_q // n_kv
+    lens_old, lens_new = [32767, 131071, 100000, 700], [1, 1, 3, 1]
+    g = torch.Generator(device=DEV).manual_seed(7)
+    scale = hd ** -0.5
+    total_pages = sum((a + b + page_size - 1) // page_size for a, b in zip(lens_old, lens_new)) + 1
+    perm = torch.randperm(total_pages, generator=torch.Generator().manual_seed(7))
+    width = max((a + b + page_size - 1) // page_size for a, b in zip(lens_old, lens_new))
+    table = torch.full((len(lens_old), width), -1, dtype=torch.int32)
+    cache = torch.full((total_pages, 2, n_kv, page_size * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    kc = cache[:, 0].view(total_pages, n_kv, page_size, hd)
+    vc = cache[:, 1].view(total_pages, n_kv, page_size // 8, hd, 8)
+    used, q_rows, want_rows = 0, [], []
+    for b, (n0, n1) in enumerate(zip(lens_old, lens_new)):
+        n = n0 + n1
+        k = torch.randn((n, n_kv, hd), generator=g, device=DEV).to(torch.bfloat16)
+        v = torch.randn((n, n_kv, hd), generator=g, device=DEV).to(torch.bfloat16)
+        q = torch.randn((n1, n_q, hd), generator=g, device=DEV).to(torch.bfloat16)
+        far = 777 if window is None else n - 8000
+        if b == 1:  # one key answers the query's head 7 (key/value head 1) loudly
+            k[far, 1] = (q[-1, 7].float() * 4.0).to(torch.bfloat16)
+        n_pages = (n + page_size - 1) // page_size
+        table[b, :n_pages] = perm[used:used + n_pages].to(torch.int32)
+        used += n_pages
+        pos = torch.arange(n, device=DEV)
+        pages, slots = table[b].to(DEV)[pos // page_size].long(), pos % page_size
+        kc[pages, :, slots, :] = k
+        vc[pages, :, slots // 8, :, slots % 8] = v
+        want = torch.empty((n1, n_q, hd), dtype=torch.float32, device=DEV)
+        qpos = torch.arange(n0, n, device=DEV).view(-1, 1)
+        ok = pos.view(1, -1) <= qpos
+        if window is not None:
+            ok = ok & (pos.view(1, -1) >= qpos - (window - 1))
+        for h in range(n_kv):  # head by head: the scores of all 48 heads at once would be large
+            scores = torch.einsum("tgd,kd->tgk", q[:, h * group:(h + 1) * group].float(), k[:, h].float()) * scale
+            probs = torch.softmax(scores.masked_fill(~ok[:, None, :], float("-inf")), dim=-1)
+            if b == 1 and h == 1:
+                assert probs[-1, 1, far] > 0.9
+            want[:, h * group:(h + 1) * group] = torch.einsum("tgk,kd->tgd", probs, v[:, h].float())
+        want_rows.append(want.reshape(n1, -1).cpu())
+        q_rows.append(q)
+    kv_lens = [a + b for a, b in zip(lens_old, lens_new)]
+    cu = [0]
+    for n in lens_new:
+        cu.append(cu[-1] + n)
+    batch = SimpleNamespace(
+        q_lens=lens_new, kv_lens=kv_lens, n_seqs=len(kv_lens), n_tokens=sum(lens_new), scratch={},
+        cu_q=torch.tensor(cu, dtype=torch.int32).to(DEV), kv_len=torch.tensor(kv_lens, dtype=torch.int32).to(DEV),
+    )
+    got = ops.paged_attention_mfma(torch.cat(q_rows), cache, table.to(DEV), batch, window, scale).cpu()
     assert torch.isfinite(got).all()
     torch.testing.assert_close(got.float(), torch.cat(want_rows), rtol=2e-2, atol=2e-2)
 

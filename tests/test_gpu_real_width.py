@@ -57,6 +57,7 @@ def test_two_layers_of_the_32b_width(dtype, graphs):
         storage.fill_pages(group, gone, float("nan"))
 
     runner.on_pages_freed = poison
+    page_use = traces.PageUse(manager)
     runner.admit("long")
     got = {"long": {}, "short": {}}
     cur = 0
@@ -78,6 +79,7 @@ def test_two_layers_of_the_32b_width(dtype, graphs):
             portions.append(Portion("short", short_toks[short_cur : short_cur + m], swant))
             wanted += [("short", short_cur + w) for w in swant]
             short_cur += m
+        page_use.note()
         logits = runner.step(portions)
         manager.check()
         assert logits.shape == (len(wanted), vocab)
@@ -89,6 +91,7 @@ def test_two_layers_of_the_32b_width(dtype, graphs):
     # the window group gave pages back while the long request ran, and took them again
     window_group = next(g.index for g in manager.groups if g.window == 8192)
     assert any(g == window_group for g, _ in freed_pages)
+    assert page_use.pages_used_again(window_group) > 0, "no page of the window group was taken again after it had been given back"
     assert manager.pages_held("long")[window_group] <= (8191 + 1 + PAGE - 1) // PAGE + 1
 
     # the plain implementation on whole sequences, float64 on the device, from the same random tensors

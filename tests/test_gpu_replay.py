@@ -62,10 +62,15 @@ def test_replay_regimes(folders, plain_cache, name, dtype, regime):
     max_tokens = traces.max_live_tokens(steps)
     page_size = (PAGE_SIZES_D if name == "tiny_d" else PAGE_SIZES)[regime]
     rep = Replayer(folders[name, dtype], dtype, max_tokens, page_size=page_size, poison_freed_pages=True)
-    outputs = traces.run_in_process(rep, steps)
+    page_use = traces.PageUse(rep.manager)
+    outputs = traces.run_in_process(rep, steps, page_use)
     got = traces.gather(steps, outputs, {k: len(v) for k, v in requests.items()}, vocab)
     compare(got, plain_for(folders, plain_cache, name, dtype), dtype, f"{name} {dtype} {regime}")
     assert rep.manager.live_requests() == []
+    if regime == "mixed":
+        # "so few pages that they are used again": in every layer group physical pages have served two requests
+        for g in rep.manager.groups:
+            assert page_use.pages_shared_between_requests(g.index) > 0, f"group {g.index} (window {g.window}): no page served two requests"
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -370,17 +370,36 @@ def test_toy_halves_rotation_and_a_norm_before_it(dtype):
                 if t is not None:
                     t.copy_(torch.nn.functional.normalize(t.float(), dim=-1).to(t.dtype))
 
+    class ElementScaledAttention(PagedAttention):
+        """A weight per element of a head on queries and keys (as the weight of a norm per head would be).  The
+        heads reach `transform_qk` in the order the kernels rotate them, so the weight is reordered once at bind."""
+
+        def tensor_specs(self):
+            from cwm_amd.parts import TensorSpec
+
+            return {**super().tensor_specs(), "qk_scale": TensorSpec((self.head_dim,), init="norm", precision="stored")}
+
+        def bind(self, tensors, runtime):
+            super().bind(tensors, runtime)
+            self.qk_scale = tensors["qk_scale"].float()[self.qk_order.to(runtime.device)]
+
+        def transform_qk(self, q, k, batch):
+            for t in (q, k):
+                if t is not None:
+                    t.copy_((t.float() * self.qk_scale).to(t.dtype))
+
     register_part("position_encoding", "toy_halves", HalvesRotary)
     register_part("mixer", "toy_unit_norm_attention", UnitNormAttention)
+    register_part("mixer", "toy_element_scaled_attention", ElementScaledAttention)
     try:
         dim, n_heads, n_kv, hd = 40, 6, 2, 16
-        for mixer_name, normalise in (("paged_attention", False), ("toy_unit_norm_attention", True)):
-            scale = 4.0 if normalise else 0.3
+        for mixer_name, normalise in (("paged_attention", False), ("toy_unit_norm_attention", True), ("toy_element_scaled_attention", "elements")):
+            scale = 4.0 if normalise is True else 0.3
             choice = PartChoice(mixer_name, {"dim": dim, "n_heads": n_heads, "n_kv_heads": n_kv, "head_dim": hd, "scale": scale, "bias": True,
                                              "position_encoding": PartChoice("toy_halves", {"head_dim": hd})})
             part = choice.build("mixer")
             runtime = Runtime(torch.device("cuda:0"), dtype)
-            host = random_tensors(part.tensor_specs(), seed=13, std=0.4, norm_init="ones", dtype=dtype)
+            host = random_tensors(part.tensor_specs(), seed=13, std=0.4, norm_init="uniform", dtype=dtype)
             part.bind({k: v.to("cuda:0") for k, v in host.items()}, runtime)
 
             n = 23
@@ -392,10 +411,13 @@ def test_toy_halves_rotation_and_a_norm_before_it(dtype):
             q = plain.linear(xd, w["wq.weight"], w["wq.bias"]).view(n, n_heads, hd)
             k = plain.linear(xd, w["wk.weight"], w["wk.bias"]).view(n, n_kv, hd)
             v = plain.linear(xd, w["wv.weight"], w["wv.bias"]).view(n, n_kv, hd)
-            if normalise:
+            if normalise is True:
                 q, k = torch.nn.functional.normalize(q, dim=-1), torch.nn.functional.normalize(k, dim=-1)
-                if dtype == torch.bfloat16:  # the hook stores what it made
-                    q, k = q.to(dtype).double(), k.to(dtype).double()
+            elif normalise == "elements":  # in the folder's order of a head's elements
+                assert not torch.equal(part.qk_order, torch.arange(hd))
+                q, k = q * w["qk_scale"], k * w["qk_scale"]
+            if normalise and dtype == torch.bfloat16:  # the hook stores what it made
+                q, k = q.to(dtype).double(), k.to(dtype).double()
             q, k = _rotate_halves(q, pos, freqs), _rotate_halves(k, pos, freqs)
             want = plain.linear(plain.attention(q, k, v, window_left=-1, scale=scale).reshape(n, -1), w["wo.weight"]).float()
             # the pairing matters: adjacent pairs give something else
@@ -423,6 +445,7 @@ def test_toy_halves_rotation_and_a_norm_before_it(dtype):
     finally:
         del POSITION_ENCODINGS["toy_halves"]
         del MIXERS["toy_unit_norm_attention"]
+        del MIXERS["toy_element_scaled_attention"]
 
 
 def test_toy_model_with_tied_head_scaled_embedding_and_two_kinds_of_norm():
