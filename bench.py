@@ -145,16 +145,17 @@ def main() -> int:
     weight_bytes = 0
     matrix_params = 0
     head_params = 0
-    embedding = model.plan.embedding_name + ".weight"
+    head_names = model.tensor_names("head")
+    embedding_only = model.tensor_names("embedding") - head_names  # tables of which a step reads one row a token
     for name, spec in model.tensor_specs().items():
         count = 1
         for n in spec.shape:
             count *= n
-        if name == embedding and not model.plan.tied_head:
+        if name in embedding_only:
             continue
         weight_bytes += count * esize
         if len(spec.shape) == 2:
-            if name == embedding or name == model.plan.head_name + ".weight":
+            if name in head_names:
                 head_params += count
             else:
                 matrix_params += count
@@ -169,7 +170,7 @@ def main() -> int:
         for spec in model.cache_specs:
             if isinstance(spec, PagedKVSpec):
                 keys = ctx if spec.window is None else min(ctx, spec.window)
-                total += batch * keys * 2 * spec.n_kv_heads * spec.head_dim * esize
+                total += batch * keys * spec.bytes_per_token(esize)
         return total
 
     def make_runner(batch, ctx, extra):

@@ -1,7 +1,9 @@
 """Device memory of the cache: one paged tensor per cache slot that keeps keys and
 values, one slot array per cache slot that keeps fixed-size state.
 
-Paged layout per slot: [num_pages, 2, n_kv_heads, page_size * head_dim]; plane 0
+A paged slot is [num_pages, *spec.page_shape(page_size)]: the cache need of the slot's mixer says how its
+page is laid out, and only that mixer's kernels look inside.  The layout of `PagedKVSpec` itself, which the
+attention kernels of this package read: [num_pages, 2, n_kv_heads, page_size * head_dim]; plane 0
 holds a page's keys as [slot, dim], plane 1 its values in blocks of VB keys as
 [slot // VB, dim, slot % VB] with VB = 8 for page sizes that are multiples of 8 and
 the whole page otherwise (8 consecutive keys of one dimension are 16 contiguous
@@ -51,11 +53,7 @@ class CacheStorage:
         for cid, spec in enumerate(manager.specs):
             if isinstance(spec, PagedKVSpec):
                 pool = manager.groups[manager.group_of_cache[cid]].pool
-                self.paged[cid] = torch.zeros(
-                    (pool.num_pages, 2, spec.n_kv_heads, manager.page_size * spec.head_dim),
-                    dtype=dtype,
-                    device=device,
-                )
+                self.paged[cid] = torch.zeros((pool.num_pages, *spec.page_shape(manager.page_size)), dtype=dtype, device=device)
             elif isinstance(spec, StateSpec):
                 self.state[cid] = torch.zeros((manager.max_requests, *spec.shape), dtype=spec.dtype, device=device)
 

@@ -1,5 +1,7 @@
+"""Typed configurations and the registry of architectures.  An architecture's own configuration class lives in
+its own module (`cwm_amd.config.llama3` for the Llama-3 dense decoder) and is not exported from here."""
+
 from .schema import ConfigError, from_dict, to_dict
-from .llama3 import Llama3DenseConfig, ScaledRoPEConfig, WindowAttentionConfig
 from .registry import (
     ARCHITECTURES,
     Architecture,
@@ -13,9 +15,6 @@ __all__ = [
     "ConfigError",
     "from_dict",
     "to_dict",
-    "Llama3DenseConfig",
-    "ScaledRoPEConfig",
-    "WindowAttentionConfig",
     "ARCHITECTURES",
     "Architecture",
     "get_architecture",

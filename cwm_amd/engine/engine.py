@@ -68,7 +68,7 @@ def pool_sizes(
     for spec in model.cache_specs:
         if isinstance(spec, PagedKVSpec):
             key = spec.retention()
-            per_page[key] = per_page.get(key, 0) + 2 * spec.n_kv_heads * spec.head_dim * page * esize
+            per_page[key] = per_page.get(key, 0) + spec.bytes_per_token(esize) * page
             span = spec.keys_kept(args.max_prefill)
             kept[key] = None if span is None else spec.pinned_keys() + span
     if not per_page:

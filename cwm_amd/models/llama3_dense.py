@@ -48,9 +48,9 @@ def build_plan(config: Llama3DenseConfig) -> ModelPlan:
             },
         )
         layers.append(
-            LayerPlan(prefix=f"layers.{i}.", block="pre_norm", norm=norm, mixer=mixer, feed_forward=feed_forward, names=names)
+            LayerPlan.standard(prefix=f"layers.{i}.", block="pre_norm", norm=norm, mixer=mixer, feed_forward=feed_forward, names=names)
         )
-    return ModelPlan(
+    return ModelPlan.standard(
         vocab_size=config.vocab_size,
         dim=config.dim,
         embedding_name="tok_embeddings",

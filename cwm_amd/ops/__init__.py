@@ -188,7 +188,7 @@ def gate_up_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
         grouped and n % 16 == 0
         and x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
         and x.shape[0] <= STREAM_EPILOGUE_ROWS and _stream_takes(x, weight)
-        and (x.shape[1] + 31) // 32 <= 16 * 12  # K fits one group of wavefronts: no split
+        and x.shape[1] <= stream_unsplit_k(x.shape[0])  # K fits one group of wavefronts: no split
     )
     tiled = x.is_cuda and x.dim() == 2 and _prefers_tile(x, weight, bias)
     if fused and not tiled:
@@ -333,6 +333,23 @@ def _compute_units(device: torch.device) -> int:
     return _cu_count[idx]
 
 
+def _stream_block_shape(m: int) -> Tuple[int, int]:
+    """(wavefronts of a block, steps of 32 along K that one wavefront keeps of x in registers) of the streaming
+    product for `m` rows, asked of the library: the kernel's register budget is stated there and nowhere else."""
+    shape = _stream_shapes.get(m)
+    if shape is None:
+        lib = _build.load("gemm_bf16_stream")
+        shape = _stream_shapes[m] = (lib.cwm_gemm_bf16_stream_waves(ctypes.c_int(m)), lib.cwm_gemm_bf16_stream_steps_per_wave(ctypes.c_int(m)))
+    return shape
+
+
+def stream_unsplit_k(m: int) -> int:
+    """The longest K that one group of wavefronts of the streaming product holds for `m` rows, so that K is not
+    split over blocks: the fused epilogues (rotation + cache write, gated activation) need that."""
+    waves, regs = _stream_block_shape(m)
+    return 32 * waves * regs
+
+
 def gemm_bf16_stream(
     x: torch.Tensor,
     weight: torch.Tensor,
@@ -364,10 +381,7 @@ def gemm_bf16_stream(
         raise KernelError(f"gemm: bias {tuple(bias.shape)} does not fit {n} outputs")
     out_dtype = out_dtype or torch.bfloat16
     lib = _build.load("gemm_bf16_stream")
-    shape = _stream_shapes.get(m)
-    if shape is None:
-        shape = _stream_shapes[m] = (lib.cwm_gemm_bf16_stream_waves(ctypes.c_int(m)), lib.cwm_gemm_bf16_stream_steps_per_wave(ctypes.c_int(m)))
-    waves, regs = shape
+    waves, regs = _stream_block_shape(m)
     steps = (k + 31) // 32
     n_tiles = (n + 15) // 16
     cus = _compute_units(x.device)
@@ -442,7 +456,7 @@ def qkv_rope_write(
         and x.shape[0] <= STREAM_EPILOGUE_ROWS
         and head_dim <= 256
         and _stream_takes(x, weight)
-        and (x.shape[1] + 31) // 32 <= 16 * 12  # K fits one group of wavefronts: no split
+        and x.shape[1] <= stream_unsplit_k(x.shape[0])  # K fits one group of wavefronts: no split
         and not _prefers_tile(x, weight, bias)
     )
     if fused:

@@ -1,12 +1,16 @@
 from .base import (
     BLOCKS,
+    EMBEDDINGS,
     FEED_FORWARDS,
+    HEADS,
     MIXERS,
     NORMS,
     POSITION_ENCODINGS,
     Block,
     CacheSpec,
+    Embedding,
     FeedForward,
+    Head,
     LayerCall,
     LayerPlan,
     Mixer,
@@ -15,16 +19,18 @@ from .base import (
     PagedKVSpec,
     Part,
     PartChoice,
+    PartSlot,
     PositionEncoding,
     Runtime,
     StateSpec,
     TensorSpec,
     register_part,
 )
-from . import norm, rope, attention, feedforward, block  # noqa: F401  (fill the registries)
+from . import norm, rope, attention, feedforward, block, embedding  # noqa: F401  (fill the registries)
 from .linear import LinearWeights
 from .norm import RMSNorm
 from .rope import NoPositionEncoding, RotaryEncoding, llama3_scale_frequencies, rotary_inverse_frequencies
 from .attention import PagedAttention
 from .feedforward import SwiGLU
 from .block import PreNormBlock
+from .embedding import LinearHead, TokenEmbedding

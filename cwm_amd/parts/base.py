@@ -11,6 +11,8 @@ Kinds of part and their registries (name -> class):
   FEED_FORWARDS       per-token transform [T, D] -> [T, D]
   POSITION_ENCODINGS  what a mixer applies to queries and keys
   BLOCKS              arrangement of the above in one layer
+  EMBEDDINGS          token ids (and whatever else of the step) -> the float32 residual stream
+  HEADS               normalised rows -> float32 logits
 """
 
 from __future__ import annotations
@@ -74,6 +76,22 @@ class PagedKVSpec:
         if self.window is None:
             return None
         return self.window - 1 + step_tokens
+
+    # What the storage, the pool sizes and the measurements ask: how a page of this cache is laid out
+    # and what a token costs.  A mixer whose cached row is not a key and a value of equal width (one
+    # compressed row a token, say) passes a subclass that answers differently; its own kernels read
+    # the pages, nothing else looks inside them.
+    def page_shape(self, page_size: int) -> Tuple[int, ...]:
+        """Shape of one page of `page_size` tokens; the storage allocates [pages, *page_shape].
+        Here: a plane of keys and a plane of values, [2, n_kv_heads, page_size * head_dim]."""
+        return (2, self.n_kv_heads, page_size * self.head_dim)
+
+    def bytes_per_token(self, element_size: int) -> int:
+        """Bytes that one cached token takes with elements of `element_size` bytes."""
+        count = 1
+        for n in self.page_shape(1):
+            count *= n
+        return count * element_size
 
 
 @dataclass(frozen=True)
@@ -171,10 +189,72 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
-class Block(Part):
-    """One layer: an arrangement of norms, a mixer and a feed-forward."""
+class Embedding(Part):
+    """What starts the residual stream."""
 
-    mixer: Mixer
+    def forward(self, batch: Any) -> torch.Tensor:
+        """The step's `StepBatch` (`tokens` int32 [T], `positions`, ...) -> float32 [T, D], a fresh tensor
+        that the layers add into."""
+        raise NotImplementedError
+
+
+class Head(Part):
+    """What turns the final norm's rows into logits."""
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """Normalised rows [R, D] in the activation type -> float32 logits [R, V]."""
+        raise NotImplementedError
+
+
+class Block(Part):
+    """One layer: an arrangement of any number of norms, mixers and feed-forwards.
+
+    The model builds the parts that the layer's plan names and calls the block's factory with them by
+    role, as keyword arguments, and with `names`, the prefix of each role's tensors:
+        BLOCKS[block](names={"norm1": "attention_norm.", ...}, norm1=<Norm>, mixer=<Mixer>, ...)
+    A subclass that hands them on to `Block.__init__` gets `tensor_specs`, `bind`, `replayable` and
+    `mixers` from here and only has to write `forward` (`replayable` is then what the parts say; a block
+    whose own `forward` does not keep to the rule of `Part.replayable` sets it to False)."""
+
+    def __init__(self, names: Mapping[str, str], **parts: Part) -> None:
+        self.names = dict(names)
+        self.parts: Dict[str, Part] = dict(parts)
+        for role in self.parts:
+            if role not in self.names:
+                raise KeyError(f"no tensor prefix is given for the block's part {role!r}")
+
+    def _own_parts(self) -> Dict[str, Part]:
+        parts = getattr(self, "parts", None)
+        if parts is None:
+            raise NotImplementedError(f"{type(self).__name__} neither calls Block.__init__ nor defines this itself")
+        return parts
+
+    @property
+    def replayable(self) -> bool:
+        parts = getattr(self, "parts", None)
+        return parts is not None and all(part.replayable for part in parts.values())
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        specs: Dict[str, TensorSpec] = {}
+        for role, part in self._own_parts().items():
+            for name, spec in part.tensor_specs().items():
+                specs[self.names[role] + name] = spec
+        return specs
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        for role, part in self._own_parts().items():
+            prefix = self.names[role]
+            part.bind({n[len(prefix):]: t for n, t in tensors.items() if n.startswith(prefix)}, runtime)
+
+    def mixers(self) -> List[Mixer]:
+        """The block's mixers in the order in which `forward` gets their caches: each has a cache slot of its
+        own per entry of the run order.  By default the mixers among the parts, in the order of the plan (a
+        block that keeps its parts itself and has one `mixer` attribute is served too)."""
+        parts = getattr(self, "parts", None)
+        if parts is None:
+            return [self.mixer]  # type: ignore[attr-defined]
+        return [part for part in parts.values() if isinstance(part, Mixer)]
 
     def forward(
         self,
@@ -186,7 +266,8 @@ class Block(Part):
     ) -> Optional[torch.Tensor]:
         """Consumes the pending residual update `delta` of the previous layer and
         returns its own, so that each residual sum is fused with the norm that
-        follows it."""
+        follows it.  `cache` is the cache view of the block's mixer; a tuple of views, in the
+        order of `mixers()`, if it has several; None if it has none."""
         raise NotImplementedError
 
 
@@ -198,6 +279,8 @@ MIXERS: Dict[str, Callable[..., Mixer]] = {}
 FEED_FORWARDS: Dict[str, Callable[..., FeedForward]] = {}
 POSITION_ENCODINGS: Dict[str, Callable[..., PositionEncoding]] = {}
 BLOCKS: Dict[str, Callable[..., Block]] = {}
+EMBEDDINGS: Dict[str, Callable[..., Embedding]] = {}
+HEADS: Dict[str, Callable[..., Head]] = {}
 
 _REGISTRIES = {
     "norm": NORMS,
@@ -205,12 +288,14 @@ _REGISTRIES = {
     "feed_forward": FEED_FORWARDS,
     "position_encoding": POSITION_ENCODINGS,
     "block": BLOCKS,
+    "embedding": EMBEDDINGS,
+    "head": HEADS,
 }
 
 
 def register_part(kind: str, name: str, factory: Callable[..., Part]) -> None:
     """Make `factory` available to architecture builders as part `name` of `kind`
-    ("norm", "mixer", "feed_forward", "position_encoding" or "block")."""
+    ("norm", "mixer", "feed_forward", "position_encoding", "block", "embedding" or "head")."""
     if kind not in _REGISTRIES:
         raise KeyError(f"unknown kind of part {kind!r}; kinds: {', '.join(_REGISTRIES)}")
     _REGISTRIES[kind][name] = factory
@@ -234,25 +319,55 @@ class PartChoice:
 # the plan of a model: data that an architecture's builder returns
 # --------------------------------------------------------------------------- #
 @dataclass(frozen=True)
-class LayerPlan:
-    """One layer: which block arrangement, which parts, and the prefixes of their
-    tensors in the model folder.
+class PartSlot:
+    """A place in a plan: the kind of part that fills it (a registry), the part chosen, and the prefix of its
+    tensors (below the layer's prefix for a layer's parts, in the model folder for the model's own)."""
 
-    The block factory is called as
-        BLOCKS[block](norm1=Norm, mixer=Mixer, norm2=Norm, feed_forward=FeedForward, names=names)
-    where `names` maps each of these four roles to the prefix of its tensors below
-    `prefix` (for instance {"norm1": "attention_norm.", "mixer": "attention.", ...}).
-    `norm` is the norm before the mixer and, unless `norm2` names another, also the one
-    before the feed-forward.  A position encoding is an argument of the mixer that applies it.
+    kind: str
+    choice: PartChoice
+    prefix: str = ""
+
+    def build(self) -> Part:
+        return self.choice.build(self.kind)
+
+
+@dataclass(frozen=True)
+class LayerPlan:
+    """One layer: which block arrangement, and its parts by role.
+
+    The roles are the block's own: the factory is called as
+        BLOCKS[block](names={role: prefix, ...}, **{role: built part, ...})
+    so a block may have any number of norms, mixers and feed-forwards under any names.  A position encoding is
+    an argument of the mixer that applies it.  Two roles that are given one prefix read the same tensors.
     """
 
     prefix: str
     block: str
-    norm: PartChoice
-    mixer: PartChoice
-    feed_forward: PartChoice
-    names: Mapping[str, str]
-    norm2: Optional[PartChoice] = None
+    parts: Mapping[str, PartSlot]
+
+    @classmethod
+    def standard(
+        cls,
+        prefix: str,
+        block: str,
+        norm: PartChoice,
+        mixer: PartChoice,
+        feed_forward: PartChoice,
+        names: Mapping[str, str],
+        norm2: Optional[PartChoice] = None,
+    ) -> "LayerPlan":
+        """The common layer of four roles: `norm1` before the `mixer`, `norm2` (`norm` again unless another is
+        named) before the `feed_forward`; `names` gives each role's prefix."""
+        return cls(
+            prefix,
+            block,
+            {
+                "norm1": PartSlot("norm", norm, names["norm1"]),
+                "mixer": PartSlot("mixer", mixer, names["mixer"]),
+                "norm2": PartSlot("norm", norm2 or norm, names["norm2"]),
+                "feed_forward": PartSlot("feed_forward", feed_forward, names["feed_forward"]),
+            },
+        )
 
 
 @dataclass(frozen=True)
@@ -267,14 +382,42 @@ class LayerCall:
 
 @dataclass(frozen=True)
 class ModelPlan:
+    """A model as data: the embedding, the layers and the order in which they run, the final norm and the
+    head, each a part chosen by name.  What the embedding does beside the table look-up (a scale, learned
+    positions) and what the head does beside the product (a cap on the logits, a bias) belongs to those
+    parts; a head that shares the embedding's table is a head whose prefix is the embedding's."""
+
     vocab_size: int
     dim: int
-    embedding_name: str
     layers: List[LayerPlan]
     run_order: List[LayerCall]
-    final_norm: PartChoice
-    final_norm_name: str
-    head_name: str  # ignored with `tied_head`
+    embedding: PartSlot
+    final_norm: PartSlot
+    head: PartSlot
     max_positions: Optional[int] = None  # the context length the configuration names (cache sizing reads it)
-    embedding_scale: Optional[float] = None  # the embedding is multiplied by it (None: as it is)
-    tied_head: bool = False  # the output projection is the embedding table; the folder holds no head tensor
+
+    @classmethod
+    def standard(
+        cls,
+        vocab_size: int,
+        dim: int,
+        embedding_name: str,
+        layers: List[LayerPlan],
+        run_order: List[LayerCall],
+        final_norm: PartChoice,
+        final_norm_name: str,
+        head_name: str,
+        max_positions: Optional[int] = None,
+    ) -> "ModelPlan":
+        """A table of token embeddings, the layers, a norm and a linear head, each under its module's name."""
+        sizes = {"vocab_size": vocab_size, "dim": dim}
+        return cls(
+            vocab_size,
+            dim,
+            layers,
+            run_order,
+            embedding=PartSlot("embedding", PartChoice("token_embedding", sizes), embedding_name + "."),
+            final_norm=PartSlot("norm", final_norm, final_norm_name + "."),
+            head=PartSlot("head", PartChoice("linear_head", sizes), head_name + "."),
+            max_positions=max_positions,
+        )

@@ -2,11 +2,11 @@
 
 from __future__ import annotations
 
-from typing import Any, Dict, Mapping, Optional
+from typing import Any, Mapping, Optional
 
 import torch
 
-from .base import Block, FeedForward, Mixer, Norm, Runtime, TensorSpec, register_part
+from .base import Block, FeedForward, Mixer, Norm, register_part
 
 
 class PreNormBlock(Block):
@@ -16,30 +16,12 @@ class PreNormBlock(Block):
     takes the previous layer's pending update and returns its own.
     """
 
-    def __init__(self, norm1: Norm, mixer: Mixer, norm2: Norm, feed_forward: FeedForward, names: Mapping[str, str]) -> None:
+    def __init__(self, names: Mapping[str, str], norm1: Norm, mixer: Mixer, norm2: Norm, feed_forward: FeedForward) -> None:
+        super().__init__(names, norm1=norm1, mixer=mixer, norm2=norm2, feed_forward=feed_forward)
         self.norm1 = norm1
         self.mixer = mixer
         self.norm2 = norm2
         self.feed_forward = feed_forward
-        self.names = dict(names)
-        self._parts = {"norm1": norm1, "mixer": mixer, "norm2": norm2, "feed_forward": feed_forward}
-
-    @property
-    def replayable(self) -> bool:
-        return all(part.replayable for part in self._parts.values())
-
-    def tensor_specs(self) -> Dict[str, TensorSpec]:
-        specs: Dict[str, TensorSpec] = {}
-        for role, part in self._parts.items():
-            for name, spec in part.tensor_specs().items():
-                specs[self.names[role] + name] = spec
-        return specs
-
-    def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
-        super().bind(tensors, runtime)
-        for role, part in self._parts.items():
-            prefix = self.names[role]
-            part.bind({n[len(prefix):]: t for n, t in tensors.items() if n.startswith(prefix)}, runtime)
 
     def forward(self, h: torch.Tensor, delta: Optional[torch.Tensor], batch: Any, cache: Any, write_cache: bool = True) -> torch.Tensor:
         x = self.norm1.forward(h, delta)

@@ -73,6 +73,7 @@ class Replayer:
         from .cache import CacheManager, CacheStorage
         from .engine import ModelRunner, load_model, random_model
         from .engine.runner import weak_callback
+        from .parts.base import PagedKVSpec
 
         if max_tokens <= 0:
             raise ValueError("--max-tokens must be positive")
@@ -92,9 +93,8 @@ class Replayer:
         if pages is not None:
             sizes = {}
             for spec in self.model.cache_specs:
-                window = getattr(spec, "window", None)
-                if hasattr(spec, "n_kv_heads"):
-                    sizes[window] = pages.get(window, num_pages)
+                if isinstance(spec, PagedKVSpec):  # pools are keyed by what the cache need keeps (its window; None: all)
+                    sizes[spec.retention()] = pages.get(spec.retention(), num_pages)
             unknown = set(pages) - set(sizes)
             if unknown:
                 raise ValueError(f"--pages names groups that the model does not have: {sorted(map(str, unknown))}; its groups: {sorted(map(str, sizes))}")

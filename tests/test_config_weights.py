@@ -77,7 +77,8 @@ def test_missing_required_key_is_named():
 
 
 def test_config_without_a_name_goes_to_the_architecture_it_fits():
-    from cwm_amd.config import ARCHITECTURES, ConfigError, Llama3DenseConfig, parse_config, register_architecture
+    from cwm_amd.config import ARCHITECTURES, ConfigError, parse_config, register_architecture
+    from cwm_amd.config.llama3 import Llama3DenseConfig
     from cwm_amd.models.llama3_dense import build_plan
 
     data = configs.get("tiny_b")
@@ -120,7 +121,8 @@ def test_load_config_errors(tmp_path):
 
 
 def test_registry_takes_another_architecture():
-    from cwm_amd.config import ARCHITECTURES, Llama3DenseConfig, get_architecture, register_architecture
+    from cwm_amd.config import ARCHITECTURES, get_architecture, register_architecture
+    from cwm_amd.config.llama3 import Llama3DenseConfig
     from cwm_amd.models.llama3_dense import build_plan
 
     register_architecture("llama3_dense_alias_for_test", Llama3DenseConfig, build_plan)

@@ -261,12 +261,12 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
         attn = PartChoice("paged_attention", {"dim": cfg.dim, "n_heads": 2, "n_kv_heads": 1, "head_dim": 16, "scale": 0.25,
                                               "window": 5, "position_encoding": PartChoice("rotary", {"head_dim": 16, "theta": 100.0})})
         layers = [
-            LayerPlan("l0.", "pre_norm", norm, PartChoice("toy_running_sum", {"dim": cfg.dim}), ff, names),
-            LayerPlan("l1.", "pre_norm", norm, attn, ff, names),
+            LayerPlan.standard("l0.", "pre_norm", norm, PartChoice("toy_running_sum", {"dim": cfg.dim}), ff, names),
+            LayerPlan.standard("l1.", "pre_norm", norm, attn, ff, names),
         ]
         # the run order names layer 1 twice (shared weights, a cache each) and ends with the toy layer again
         order = [LayerCall(0), LayerCall(1), LayerCall(1), LayerCall(0)]
-        return ModelPlan(cfg.vocab_size, cfg.dim, "emb", layers, order, norm, "final", "head")
+        return ModelPlan.standard(cfg.vocab_size, cfg.dim, "emb", layers, order, norm, "final", "head")
 
     register_part("mixer", "toy_running_sum", RunningSumMixer)
     register_architecture("toy_state_model", ToyConfig, toy_plan)

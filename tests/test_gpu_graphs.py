@@ -224,8 +224,8 @@ def test_a_part_from_outside_opts_into_captured_steps(says_so):
                                                                  "position_encoding": rope})
         names = {"norm1": "n1.", "mixer": "attn.", "norm2": "n2.", "feed_forward": "ff."}
         norm = PartChoice("rmsnorm", {"dim": cfg.dim, "eps": 1e-5})
-        layer = LayerPlan("l0.", "pre_norm", norm, attn, PartChoice("swiglu", {"dim": cfg.dim, "hidden_dim": 48}), names)
-        return ModelPlan(cfg.vocab_size, cfg.dim, "emb", [layer], [LayerCall(0)], norm, "final", "head")
+        layer = LayerPlan.standard("l0.", "pre_norm", norm, attn, PartChoice("swiglu", {"dim": cfg.dim, "hidden_dim": 48}), names)
+        return ModelPlan.standard(cfg.vocab_size, cfg.dim, "emb", [layer], [LayerCall(0)], norm, "final", "head")
 
     register_part("mixer", "toy_unit_norm_attention_for_graphs", UnitNormAttention)
     register_architecture("toy_graph_model", ToyConfig, toy_plan)

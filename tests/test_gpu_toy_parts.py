@@ -111,8 +111,8 @@ def test_toy_routed_feed_forward_registers_builds_and_steps():
         names = {"norm1": "n1.", "mixer": "attn.", "norm2": "n2.", "feed_forward": "ff."}
         routed = PartChoice("toy_top1_experts", {"dim": cfg.dim, "hidden_dim": 24, "n_experts": cfg.n_experts})
         dense = PartChoice("swiglu", {"dim": cfg.dim, "hidden_dim": 40})
-        layers = [LayerPlan("l0.", "pre_norm", norm, attn, routed, names), LayerPlan("l1.", "pre_norm", norm, attn, dense, names)]
-        return ModelPlan(cfg.vocab_size, cfg.dim, "emb", layers, [LayerCall(0), LayerCall(1)], norm, "final", "head")
+        layers = [LayerPlan.standard("l0.", "pre_norm", norm, attn, routed, names), LayerPlan.standard("l1.", "pre_norm", norm, attn, dense, names)]
+        return ModelPlan.standard(cfg.vocab_size, cfg.dim, "emb", layers, [LayerCall(0), LayerCall(1)], norm, "final", "head")
 
     register_part("feed_forward", "toy_top1_experts", Top1Experts)
     register_architecture("toy_routed_model", ToyConfig, toy_plan)
@@ -197,9 +197,9 @@ def test_run_order_lets_a_layer_read_another_layers_cache(dtype):
             return PartChoice("paged_attention", {"dim": cfg.dim, "n_heads": n_heads, "n_kv_heads": n_kv, "head_dim": hd,
                                                   "scale": hd**-0.5, "window": w, "position_encoding": rope})
 
-        layers = [LayerPlan(f"l{i}.", "pre_norm", norm, attn(w), ff, names) for i, w in enumerate((window, None, window))]
+        layers = [LayerPlan.standard(f"l{i}.", "pre_norm", norm, attn(w), ff, names) for i, w in enumerate((window, None, window))]
         order = [LayerCall(0), LayerCall(1), LayerCall(2, cache_of=0)]
-        return ModelPlan(cfg.vocab_size, cfg.dim, "emb", layers, order, norm, "final", "head")
+        return ModelPlan.standard(cfg.vocab_size, cfg.dim, "emb", layers, order, norm, "final", "head")
 
     register_architecture("toy_shared_cache_model", ToyConfig, toy_plan)
     try:
@@ -454,7 +454,7 @@ def test_toy_model_with_tied_head_scaled_embedding_and_two_kinds_of_norm():
     layer, float32, against the same computation from the plain parts."""
     from cwm_amd.config import ARCHITECTURES, parse_config, register_architecture
     from cwm_amd.models import Model
-    from cwm_amd.parts import LayerCall, LayerPlan, ModelPlan, PartChoice, Runtime
+    from cwm_amd.parts import LayerCall, LayerPlan, ModelPlan, PartChoice, PartSlot, Runtime
     from cwm_amd.weights import random_tensors
 
     @dataclass(frozen=True)
@@ -470,17 +470,21 @@ def test_toy_model_with_tied_head_scaled_embedding_and_two_kinds_of_norm():
         attn = PartChoice("paged_attention", {"dim": cfg.dim, "n_heads": n_heads, "n_kv_heads": n_kv, "head_dim": hd, "scale": hd**-0.5,
                                               "position_encoding": rope})
         names = {"norm1": "n1.", "mixer": "attn.", "norm2": "n2.", "feed_forward": "ff."}
-        layer = LayerPlan("l0.", "pre_norm", PartChoice("rmsnorm", {"dim": cfg.dim, "eps": eps1}), attn,
-                          PartChoice("swiglu", {"dim": cfg.dim, "hidden_dim": 40}), names,
-                          norm2=PartChoice("rmsnorm", {"dim": cfg.dim, "eps": eps2}))
-        return ModelPlan(cfg.vocab_size, cfg.dim, "emb", [layer], [LayerCall(0)], PartChoice("rmsnorm", {"dim": cfg.dim, "eps": eps1}),
-                         "final", "unused", embedding_scale=emb_scale, tied_head=True)
+        layer = LayerPlan.standard("l0.", "pre_norm", PartChoice("rmsnorm", {"dim": cfg.dim, "eps": eps1}), attn,
+                                   PartChoice("swiglu", {"dim": cfg.dim, "hidden_dim": 40}), names,
+                                   norm2=PartChoice("rmsnorm", {"dim": cfg.dim, "eps": eps2}))
+        sizes = {"vocab_size": cfg.vocab_size, "dim": cfg.dim}
+        # the scale is an argument of the embedding part; the head is tied by reading the embedding's tensors
+        return ModelPlan(cfg.vocab_size, cfg.dim, [layer], [LayerCall(0)],
+                         embedding=PartSlot("embedding", PartChoice("token_embedding", {**sizes, "scale": emb_scale}), "emb."),
+                         final_norm=PartSlot("norm", PartChoice("rmsnorm", {"dim": cfg.dim, "eps": eps1}), "final."),
+                         head=PartSlot("head", PartChoice("linear_head", sizes), "emb."))
 
     register_architecture("toy_tied_model", ToyConfig, toy_plan)
     try:
         arch, cfg = parse_config({"architecture": "toy_tied_model", "dim": 32, "vocab_size": 59})
         model = Model(arch.build_plan(cfg))
-        assert "unused.weight" not in model.tensor_specs() and "emb.weight" in model.tensor_specs()
+        assert {n for n in model.tensor_specs() if not n.startswith("l0.")} == {"emb.weight", "final.weight"}  # no head tensor of its own
         runtime = Runtime(torch.device("cuda:0"), torch.float32)
         host = random_tensors(model.tensor_specs(), seed=6, std=0.3, norm_init="uniform", dtype=torch.float32)
         model.bind({k: v.to("cuda:0") for k, v in host.items()}, runtime)
@@ -521,7 +525,7 @@ def test_toy_norm_and_toy_block_arrangement_register_build_and_step():
     from cwm_amd import ops
     from cwm_amd.config import ARCHITECTURES, parse_config, register_architecture
     from cwm_amd.models import Model
-    from cwm_amd.parts import Block, LayerCall, LayerPlan, ModelPlan, Norm, PartChoice, Runtime, TensorSpec, register_part
+    from cwm_amd.parts import Block, LayerCall, LayerPlan, ModelPlan, Norm, PartChoice, PartSlot, Runtime, TensorSpec, register_part
     from cwm_amd.weights import random_tensors
 
     class CentredNorm(Norm):
@@ -547,20 +551,9 @@ def test_toy_norm_and_toy_block_arrangement_register_build_and_step():
     class ParallelBlock(Block):
         """h += mixer(norm(h)) + feed_forward(norm(h)): one norm, two readers."""
 
-        def __init__(self, norm1, mixer, norm2, feed_forward, names):
-            self.norm, self.mixer, self.feed_forward, self.names = norm1, mixer, feed_forward, dict(names)
-
-        def _parts(self):
-            return {"norm1": self.norm, "mixer": self.mixer, "feed_forward": self.feed_forward}
-
-        def tensor_specs(self):
-            return {self.names[role] + n: s for role, part in self._parts().items() for n, s in part.tensor_specs().items()}
-
-        def bind(self, tensors, runtime):
-            super().bind(tensors, runtime)
-            for role, part in self._parts().items():
-                prefix = self.names[role]
-                part.bind({n[len(prefix):]: t for n, t in tensors.items() if n.startswith(prefix)}, runtime)
+        def __init__(self, names, norm, mixer, feed_forward):
+            super().__init__(names, norm=norm, mixer=mixer, feed_forward=feed_forward)  # tensors and bind come from Block
+            self.norm, self.mixer, self.feed_forward = norm, mixer, feed_forward
 
         def forward(self, h, delta, batch, cache, write_cache=True):
             x = self.norm.forward(h, delta)
@@ -583,15 +576,18 @@ def test_toy_norm_and_toy_block_arrangement_register_build_and_step():
     def toy_plan(cfg):
         rope = PartChoice("rotary", {"head_dim": hd, "theta": theta})
         norm = PartChoice("toy_centred", {"dim": cfg.dim, "eps": eps})
-        names = {"norm1": "ln.", "mixer": "attn.", "norm2": "unused.", "feed_forward": "ff."}
+        attn = PartChoice("paged_attention", {"dim": cfg.dim, "n_heads": n_heads, "n_kv_heads": n_kv, "head_dim": hd, "scale": hd**-0.5,
+                                              "position_encoding": rope})
+        # the layer's roles are the block's own: one norm, a mixer, a feed-forward
         layers = [
-            LayerPlan(f"l{i}.", "toy_parallel", norm,
-                      PartChoice("paged_attention", {"dim": cfg.dim, "n_heads": n_heads, "n_kv_heads": n_kv, "head_dim": hd, "scale": hd**-0.5,
-                                                     "position_encoding": rope}),
-                      PartChoice("swiglu", {"dim": cfg.dim, "hidden_dim": hidden}), names)
+            LayerPlan(f"l{i}.", "toy_parallel", {
+                "norm": PartSlot("norm", norm, "ln."),
+                "mixer": PartSlot("mixer", attn, "attn."),
+                "feed_forward": PartSlot("feed_forward", PartChoice("swiglu", {"dim": cfg.dim, "hidden_dim": hidden}), "ff."),
+            })
             for i in range(2)
         ]
-        return ModelPlan(cfg.vocab_size, cfg.dim, "emb", layers, [LayerCall(0), LayerCall(1)], norm, "final", "head")
+        return ModelPlan.standard(cfg.vocab_size, cfg.dim, "emb", layers, [LayerCall(0), LayerCall(1)], norm, "final", "head")
 
     register_architecture("toy_parallel_model", ToyConfig, toy_plan)
     try:
@@ -599,7 +595,7 @@ def test_toy_norm_and_toy_block_arrangement_register_build_and_step():
         model = Model(arch.build_plan(cfg))
         assert not model.replayable  # the toy parts do not say that their steps may be captured: every step is launched
         specs = model.tensor_specs()
-        assert "l1.ln.bias" in specs and not any(n.startswith("l0.unused.") for n in specs)
+        assert "l1.ln.bias" in specs and sorted({n.split(".")[1] for n in specs if n.startswith("l0.")}) == ["attn", "ff", "ln"]
         runtime = Runtime(torch.device("cuda:0"), torch.float32)
         host = random_tensors(specs, seed=12, std=0.3, norm_init="uniform", dtype=torch.float32)
         model.bind({k: v.to("cuda:0") for k, v in host.items()}, runtime)
