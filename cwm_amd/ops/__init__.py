@@ -1107,3 +1107,50 @@ __all__ = [
     "unpack_sampled",
     "token_logprobs",
 ]
+
+
+# --------------------------------------------------------------------------- #
+# what the GPU at hand reaches (for the measurement program; nothing on the model's path)
+def measure_read_rate(buffer: torch.Tensor, window_bytes: int, launches: int, blocks: int) -> float:
+    """GB/s at which a kernel that only reads gets through `window_bytes` of `buffer` (uint8, on the device):
+    `launches` launches back to back, each on the next window of the buffer (so that, with a buffer several times
+    the last-level cache, no launch finds its bytes cached), timed by events around all of them."""
+    _need_gpu(buffer)
+    if buffer.dtype != torch.uint8 or not buffer.is_contiguous() or window_bytes % 16 != 0 or not 0 < window_bytes <= buffer.numel():
+        raise KernelError("measure_read_rate takes a contiguous uint8 buffer and a window that is a multiple of 16 bytes within it")
+    lib = _build.load("ceilings")
+    windows = max(1, buffer.numel() // window_bytes)
+    base = buffer.data_ptr()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    stream = _stream()
+    for timed in (False, True):
+        if timed:
+            start.record()
+        for i in range(launches if timed else 2):
+            offset = (i % windows) * window_bytes
+            _check(lib, lib.cwm_ceiling_read(ctypes.c_void_p(base + offset), ctypes.c_long(window_bytes), ctypes.c_int(blocks), ctypes.c_void_p(0), stream))
+        if timed:
+            end.record()
+        torch.cuda.synchronize(buffer.device)
+    return window_bytes * launches / (start.elapsed_time(end) * 1e-3) / 1e9
+
+
+def measure_mfma_rate(device: torch.device, blocks: int, rounds: int, launches: int = 3, shape: int = 16, seed: float = 1.0) -> float:
+    """PFLOP/s of the bfloat16 matrix instruction (`shape` 16: 16x16x32, 32: 32x32x16; float32 sums) issued from
+    registers by `blocks` blocks of four wavefronts, `rounds` rounds of eight independent instructions each, on
+    operands of `seed` times small varied numbers (0: all zeros, which costs the least power)."""
+    lib = _build.load("ceilings")
+    lib.cwm_ceiling_mfma_flops.restype = ctypes.c_double
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    with torch.cuda.device(device):
+        stream = _stream()
+        for timed in (False, True):
+            if timed:
+                start.record()
+            for _ in range(launches if timed else 1):
+                _check(lib, lib.cwm_ceiling_mfma(ctypes.c_int(blocks), ctypes.c_int(rounds), ctypes.c_int(shape), ctypes.c_float(seed), ctypes.c_void_p(0), stream))
+            if timed:
+                end.record()
+            torch.cuda.synchronize(device)
+    flops = lib.cwm_ceiling_mfma_flops(ctypes.c_int(blocks), ctypes.c_int(rounds)) * launches
+    return flops / (start.elapsed_time(end) * 1e-3) / 1e15

@@ -54,6 +54,7 @@ SOURCES: Dict[str, Tuple[Mapping[str, int], ...]] = {
     "sampling": ({},),
     "gemm_bf16_stream": ({},),
     "gemm_bf16_tile": ({},),
+    "ceilings": ({},),
     "attention_mfma": tuple({"HEAD_DIM": hd} for hd in (16, 32, 48, 64, 80, 96, 128, 256)),
 }
 
