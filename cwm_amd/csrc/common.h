@@ -97,6 +97,7 @@ union Frag8 {
   uint4 u;
   bf16x8 v;
   uint16_t h[8];
+  uint32_t __attribute__((ext_vector_type(4))) w;  // the same 16 bytes as a vector the non-temporal load builtin takes
 };
 
 // Direct load from global memory into LDS (global_load_lds_dwordx4): every lane's 16 bytes at

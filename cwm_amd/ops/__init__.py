@@ -177,7 +177,9 @@ def silu_mul(gate_up: torch.Tensor, out_dtype: Optional[torch.dtype] = None, gro
     return out
 
 
-def gate_up_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], grouped: bool) -> torch.Tensor:
+def gate_up_silu(
+    x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], grouped: bool, streamed: Optional[torch.Tensor] = None
+) -> torch.Tensor:
     """silu(x Wg^T) * (x Wu^T) for the joined weight [2F, D] of a gated feed-forward
     (cwm/fastgen/forward.py:776-781): rows Wg then Wu, or, with `grouped`, alternating
     in groups of 8.  A grouped weight lets a decode batch in bfloat16 finish the
@@ -192,10 +194,10 @@ def gate_up_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
     )
     tiled = x.is_cuda and x.dim() == 2 and _prefers_tile(x, weight, bias)
     if fused and not tiled:
-        return gemm_bf16_stream(x, weight, bias, torch.bfloat16, glu=True)
+        return gemm_bf16_stream(x, weight, bias, torch.bfloat16, glu=True, streamed=streamed)
     if tiled and grouped and x.shape[0] <= TILE_ROWS:
         return gemm_bf16_tile(x, weight, None, torch.bfloat16, glu=True)
-    return silu_mul(linear(x, weight, bias, partials_ok=True), out_dtype=x.dtype, grouped=grouped)
+    return silu_mul(linear(x, weight, bias, partials_ok=True, streamed=streamed), out_dtype=x.dtype, grouped=grouped)
 
 
 # --------------------------------------------------------------------------- #
@@ -302,6 +304,7 @@ def linear(
     bias: Optional[torch.Tensor] = None,
     out_dtype: Optional[torch.dtype] = None,
     partials_ok: bool = False,
+    streamed: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """y = x W^T (+ b).  cwm/fastgen/forward.py:593-606.
 
@@ -309,14 +312,15 @@ def linear(
     rows of float32 on the weight-streaming one, whose sums differ from the other's by rounding).
     bfloat16 activations and weights: matrix cores with float32 accumulation, the
     library product for many rows.  With `partials_ok` the result may be float32
-    partial sums [P, M, N] that the caller adds (see `add_rmsnorm`).
+    partial sums [P, M, N] that the caller adds (see `add_rmsnorm`).  `streamed`: the weight's
+    streaming copy (`stream_layout`), which the products of few rows read instead where there is one.
     """
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.float32 or weight.dtype == torch.float32:
         if x.is_cuda and _f32_stream_takes(x, weight):
             return gemm_f32_stream(x, weight, bias, out_dtype, partials_ok)
         return gemm_f32(x, weight, bias, out_dtype)
-    return gemm_bf16(x, weight, bias, out_dtype, partials_ok)
+    return gemm_bf16(x, weight, bias, out_dtype, partials_ok, streamed)
 
 
 STREAM_MAX_ROWS = 64
@@ -350,6 +354,20 @@ def stream_unsplit_k(m: int) -> int:
     return 32 * waves * regs
 
 
+def stream_layout(weight: torch.Tensor) -> torch.Tensor:
+    """The streaming copy of a bfloat16 matrix W [N, K]: [tiles of 16 rows, steps of 32 columns, 64, 8], lane
+    16 j + r of a step holding W[16 tile + r][32 step + 8 j ..+8] (one operand of the matrix instruction), zeros
+    past N and K.  The streaming product reads it 1 KB a wavefront's load, every cache line once."""
+    _need_gpu(weight)
+    if weight.dtype != torch.bfloat16 or weight.dim() != 2 or weight.stride(1) != 1:
+        raise KernelError("a streaming copy is made of a bfloat16 matrix with contiguous rows")
+    n, k = weight.shape
+    out = torch.empty((-(-n // 16), -(-k // 32), 64, 8), dtype=torch.bfloat16, device=weight.device)
+    lib = _build.load("gemm_bf16_stream")
+    _check(lib, lib.cwm_gemm_bf16_stream_copy(_ptr(weight), ctypes.c_long(weight.stride(0)), _ptr(out), ctypes.c_int(n), ctypes.c_int(k), _stream()))
+    return out
+
+
 def gemm_bf16_stream(
     x: torch.Tensor,
     weight: torch.Tensor,
@@ -358,9 +376,12 @@ def gemm_bf16_stream(
     partials_ok: bool = False,
     rope: Optional[tuple] = None,
     glu: bool = False,
+    streamed: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """bfloat16 x [M <= 64, K] @ weight[N, K]^T with persistent blocks that keep x in
-    registers and stream the weight once.  Returns [M, N]; with `partials_ok` it may
+    registers and stream the weight once.  `streamed` is the matrix's streaming copy
+    (`stream_layout(weight)`); with it the kernel reads that copy, in whole cache lines and past the
+    caches, instead of `weight`.  Returns [M, N]; with `partials_ok` it may
     return float32 partial sums [P, M, N] of a split K for the caller to add (the
     residual-add + RMSNorm kernel takes them).  `rope`
     (positions, seq_of_token, inv_freq, cache, block_table, n_q_heads, n_kv_heads,
@@ -398,14 +419,20 @@ def gemm_bf16_stream(
         out = torch.empty((m, n // 2 if glu else n), dtype=out_dtype, device=x.device)
     else:
         out = torch.empty((k_split, m, n), dtype=torch.float32, device=x.device)
+    if streamed is not None:
+        if streamed.shape != (n_tiles, steps, 64, 8) or streamed.dtype != torch.bfloat16 or not streamed.is_contiguous() or streamed.device != x.device:
+            raise KernelError(f"the streaming copy of a [{n}, {k}] matrix is bfloat16 [{n_tiles}, {steps}, 64, 8], not {tuple(streamed.shape)}")
+        w_ptr, w_stride = _ptr(streamed), ctypes.c_long(steps * 512)
+    else:
+        w_ptr, w_stride = _ptr(weight), ctypes.c_long(weight.stride(0) if n > 1 else k)
     _check(
         lib,
         lib.cwm_gemm_bf16_stream(
-            _ptr(x), ctypes.c_long(x.stride(0) if m > 1 else x.shape[1]), _ptr(weight), ctypes.c_long(weight.stride(0) if n > 1 else k),
+            _ptr(x), ctypes.c_long(x.stride(0) if m > 1 else x.shape[1]), w_ptr, w_stride,
             _ptr(out), ctypes.c_int(_code(out.dtype)), ctypes.c_long(out.shape[-1]), ctypes.c_long(m * n),
             _ptr(bias), ctypes.c_int(_code(bias.dtype) if bias is not None else F32),
             ctypes.c_int(m), ctypes.c_int(n), ctypes.c_int(k), ctypes.c_int(k_split), ctypes.c_int(blocks),
-            *_rope_args(rope), ctypes.c_int(int(glu)), _stream(),
+            *_rope_args(rope), ctypes.c_int(int(glu)), ctypes.c_int(int(streamed is not None)), _stream(),
         ),
     )
     if k_split > 1 and not partials_ok:
@@ -439,6 +466,7 @@ def qkv_rope_write(
     cache: torch.Tensor,
     block_table: torch.Tensor,
     seq_of_token: torch.Tensor,
+    streamed: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """The joined q/k/v projection of x [T, D] (weight [(Hq + 2 Hkv) * hd, D]), the
     rotation of its q and k columns by each token's position, and the write of the
@@ -471,9 +499,9 @@ def qkv_rope_write(
             raise KernelError("positions and seq_of_token must be [T], block_table [B, W]")
         return gemm_bf16_stream(
             x, weight, bias, torch.bfloat16,
-            rope=(positions, seq_of_token, inv_freq, cache, block_table, n_q_heads, n_kv_heads, head_dim),
+            rope=(positions, seq_of_token, inv_freq, cache, block_table, n_q_heads, n_kv_heads, head_dim), streamed=streamed,
         )
-    qkv = linear(x, weight, bias, partials_ok=True)
+    qkv = linear(x, weight, bias, partials_ok=True, streamed=streamed)
     if qkv.dim() == 3:
         # partial sums of a split K: added by the rotation kernel where it can, else by a kernel of their own
         if x.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and head_dim % 8 == 0 and head_dim <= 256:
@@ -671,6 +699,7 @@ def gemm_bf16(
     bias: Optional[torch.Tensor] = None,
     out_dtype: Optional[torch.dtype] = None,
     partials_ok: bool = False,
+    streamed: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """bfloat16 x [M, K] @ bfloat16 weight[N, K]^T, float32 accumulation.
 
@@ -689,7 +718,7 @@ def gemm_bf16(
     if _prefers_tile(x, weight, bias):
         return gemm_bf16_tile(x, weight, None, out_dtype, partials_ok)
     if m <= STREAM_MAX_ROWS:
-        return gemm_bf16_stream(x, weight, bias, out_dtype, partials_ok)
+        return gemm_bf16_stream(x, weight, bias, out_dtype, partials_ok, streamed=streamed)
     if out_dtype == torch.float32:
         y = torch.mm(x, weight.t(), out_dtype=torch.float32)  # bfloat16 operands, float32 sums written as they are
         return y if bias is None else y + bias.float()

@@ -95,8 +95,8 @@ class PagedAttention(Mixer):
                     biases[n] = biases[n][rows]
         elif pairing != "adjacent":
             raise ValueError(f"rotary pairing {pairing!r}: 'adjacent' and 'halves' are known")
-        self.qkv = LinearWeights.joined([weights[n] for n in names], [biases[n] for n in names])
-        self.wo = LinearWeights(tensors["wo.weight"])
+        self.qkv = LinearWeights.joined([weights[n] for n in names], [biases[n] for n in names], stream_copy=runtime.stream_copies)
+        self.wo = LinearWeights(tensors["wo.weight"], stream_copy=runtime.stream_copies)
         # a subclass that changes queries and keys between projection and rotation cannot use the fused product
         self._plain_projection = type(self).transform_qk is not PagedAttention.transform_qk
 
@@ -128,7 +128,7 @@ class PagedAttention(Mixer):
         if write_cache and not self._plain_projection:
             qkv = ops.qkv_rope_write(
                 x, self.qkv.weight, self.qkv.bias, self.n_heads, self.n_kv_heads, hd,
-                batch.positions, table, cache.cache, cache.block_table, batch.seq_of_token,
+                batch.positions, table, cache.cache, cache.block_table, batch.seq_of_token, streamed=self.qkv.streamed,
             )
             q = qkv[:, :q_out].unflatten(1, (self.n_heads, hd))
         else:

@@ -115,6 +115,10 @@ class Runtime:
 
     device: torch.device
     act_dtype: torch.dtype
+    # Whether matrices keep, beside the row-major tensor that products of many rows read, a second copy laid out
+    # for the weight-streaming product of a decode step (`ops.stream_layout`): twice the memory for the matrices,
+    # about a tenth less time to stream them.  Whoever loads the model decides, from the memory there is.
+    stream_copies: bool = False
 
     @property
     def is_float32(self) -> bool:

@@ -48,7 +48,7 @@ class LinearHead(Head):
 
     def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
         super().bind(tensors, runtime)
-        self.weights = LinearWeights(tensors["weight"])
+        self.weights = LinearWeights(tensors["weight"], stream_copy=runtime.stream_copies)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self.weights(x, out_dtype=torch.float32)

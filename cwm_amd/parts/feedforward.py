@@ -36,15 +36,16 @@ class SwiGLU(FeedForward):
         # finishes silu(gate) * up in the product's epilogue
         self.grouped = self.hidden_dim % 8 == 0
         self.gate_up = LinearWeights.joined(
-            [tensors["w1.weight"], tensors["w3.weight"]], [None, None], group=8 if self.grouped else None
+            [tensors["w1.weight"], tensors["w3.weight"]], [None, None], group=8 if self.grouped else None,
+            stream_copy=runtime.stream_copies,
         )
-        self.down = LinearWeights(tensors["w2.weight"])
+        self.down = LinearWeights(tensors["w2.weight"], stream_copy=runtime.stream_copies)
 
     def forward(self, x: torch.Tensor, batch: Any) -> torch.Tensor:
         # the result (or partial sums of it) is added into the residual by the next norm.  (Forming
         # silu(gate) * up inside the down product was tried: every block recomputes it, which costs
         # more than the kernel it saves.)
-        hidden = ops.gate_up_silu(x, self.gate_up.weight, self.gate_up.bias, self.grouped)
+        hidden = ops.gate_up_silu(x, self.gate_up.weight, self.gate_up.bias, self.grouped, streamed=self.gate_up.streamed)
         return self.down(hidden, partials_ok=True)
 
 

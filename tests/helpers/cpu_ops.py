@@ -49,11 +49,11 @@ def silu_mul(gate_up, out_dtype=None, grouped=False):
     return (g * torch.sigmoid(g) * u).to(gate_up.dtype)
 
 
-def gate_up_silu(x, weight, bias, grouped):
+def gate_up_silu(x, weight, bias, grouped, streamed=None):
     return silu_mul(linear(x, weight, bias), grouped=grouped)
 
 
-def linear(x, weight, bias=None, out_dtype=None, partials_ok=False):
+def linear(x, weight, bias=None, out_dtype=None, partials_ok=False, streamed=None):
     y = x.float() @ weight.float().T
     if bias is not None:
         y = y + bias.float()
@@ -93,7 +93,7 @@ def rope_kv_write(q, k, v, positions, inv_freq, cache=None, block_table=None, se
         cache_layout.write_kv(cache, page, slot, k[t], v[t], hd)
 
 
-def qkv_rope_write(x, weight, bias, n_q_heads, n_kv_heads, head_dim, positions, inv_freq, cache, block_table, seq_of_token):
+def qkv_rope_write(x, weight, bias, n_q_heads, n_kv_heads, head_dim, positions, inv_freq, cache, block_table, seq_of_token, streamed=None):
     qkv = linear(x, weight, bias)
     q_out, kv_out = n_q_heads * head_dim, n_kv_heads * head_dim
     q = qkv[:, :q_out].unflatten(1, (n_q_heads, head_dim))

@@ -1040,6 +1040,54 @@ def test_gemm_bf16_stream(out_dtype, m, n, k):
     assert torch.equal(got2, got)
 
 
+def _stream_layout_by_hand(w):
+    """The streaming copy as its definition reads: [tiles of 16 rows, steps of 32 columns, 64, 8], lane 16 j + r
+    of a step holding W[16 tile + r][32 step + 8 j ..+8], zeros past the matrix."""
+    n, k = w.shape
+    tiles, steps = -(-n // 16), -(-k // 32)
+    padded = torch.zeros((tiles * 16, steps * 32), dtype=w.dtype)
+    padded[:n, :k] = w
+    return padded.view(tiles, 16, steps, 4, 8).permute(0, 2, 3, 1, 4).reshape(tiles, steps, 64, 8).contiguous()
+
+
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(1, 263, 120), (8, 6144, 6144), (5, 64, 64), (16, 509, 296), (7, 130, 8), (3, 1000, 21504), (16, 48, 4104), (2, 7, 40),
+                                   (33, 1000, 21504 // 4), (64, 48, 4104)])
+def test_gemm_bf16_stream_from_the_streaming_copy(out_dtype, m, n, k):
+    """The product from the matrix's streaming copy: the copy is what its definition says (also for sizes that
+    fill no whole tile or step, and for a view with a wider row stride), and the product from it gives the bits
+    of the product from the row-major matrix: the same values meet in the same order."""
+    from cwm_amd import ops
+
+    a = rnd((m, k), torch.bfloat16, 16).to(DEV)
+    w = rnd((n, k), torch.bfloat16, 17, 0.05)
+    b = rnd((n,), torch.bfloat16, 18).to(DEV)
+    copy = ops.stream_layout(w.to(DEV))
+    assert torch.equal(copy.cpu(), _stream_layout_by_hand(w))
+    wide = torch.zeros((n, k + 16), dtype=torch.bfloat16)
+    wide[:, 8 : 8 + k] = w
+    assert torch.equal(ops.stream_layout(wide.to(DEV)[:, 8 : 8 + k]).cpu(), copy.cpu())
+    for partials_ok in (False, True):
+        plain = ops.gemm_bf16_stream(a, w.to(DEV), b, out_dtype=out_dtype, partials_ok=partials_ok)
+        # the row-major matrix is not read: a matrix of NaN in its place changes nothing
+        nan = torch.full((n, k), float("nan"), dtype=torch.bfloat16, device=DEV)
+        got = ops.gemm_bf16_stream(a, nan, b, out_dtype=out_dtype, partials_ok=partials_ok, streamed=copy)
+        assert got.shape == plain.shape and torch.equal(got, plain)
+    with pytest.raises(ops.KernelError, match="streaming copy"):
+        ops.gemm_bf16_stream(a, w.to(DEV), b, out_dtype=out_dtype, streamed=copy[:, :-1].contiguous() if copy.shape[1] > 1 else copy[:-1].contiguous())
+
+
+@pytest.mark.parametrize("m,f,k", [(1, 24, 64), (8, 21504 // 8, 6144 // 4), (16, 296, 120), (5, 8, 8)])
+def test_gated_epilogue_from_the_streaming_copy(m, f, k):
+    from cwm_amd import ops
+
+    x = rnd((m, k), torch.bfloat16, 21).to(DEV)
+    w = rnd((2 * f, k), torch.bfloat16, 22, 0.1).to(DEV)
+    plain = ops.gate_up_silu(x, w, None, True)
+    got = ops.gate_up_silu(x, torch.full_like(w, float("nan")), None, True, streamed=ops.stream_layout(w))
+    assert torch.equal(got, plain)
+
+
 def test_add_rmsnorm_takes_partial_sums():
     from cwm_amd import ops
 
@@ -1093,6 +1141,10 @@ def test_qkv_rope_write_fused_equals_separate(n_q, n_kv, hd, page_size, dim, bia
     assert torch.equal(fused, qkv)
     assert torch.equal(caches[0], caches[1])
     assert caches[0].abs().sum() > 0
+    # and from the matrix's streaming copy (the row-major matrix is then not read)
+    third = torch.zeros_like(caches[0])
+    streamed = ops.qkv_rope_write(x, torch.full_like(w, float("nan")), b, n_q, n_kv, hd, positions, inv_freq, third, table, seq, streamed=ops.stream_layout(w))
+    assert torch.equal(streamed, fused) and torch.equal(third, caches[0])
 
 
 @pytest.mark.parametrize(
