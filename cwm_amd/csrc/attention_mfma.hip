@@ -53,6 +53,7 @@ CWM_DEFINE_ERROR_API
 #define PARTIAL_STRIDE (HEAD_DIM + 4)  // max and sum after the output; keeps rows 16-byte aligned
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) { return pack2_bf16(lo, hi); }
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // One row's share of a 32-key tile of scores: masks (only where a tile reaches past some
 // row's keys), the probabilities as the matrix-core B operand, and the factor that rescales
@@ -122,13 +123,27 @@ __device__ __forceinline__ bool span_lacks_page(const int* __restrict__ table, i
 }
 
 // work item: {sequence, first row, first key, end key (exclusive), partial slot or -1, unused}
-// One wavefront per (work item, key/value head); RT: 16-row tiles that a wavefront takes from
-// the item's first row on.  Decoded tokens and short portions run with RT = 1 (sequences with
-// many rows go to the kernel further down that shares keys and values through LDS).
-// UNIFORM_WAVE: the wavefront's index is declared the same for all 64 lanes, so its work item
-// and lengths are loaded and held as scalars: a shorter start, which items of few keys (64 or
-// 128) feel; items of 256 keys run faster from the code that the compiler makes without it.
-template <int RT, bool UNIFORM_WAVE>
+// A block of four wavefronts (a team) per (work item, key/value head), on the 16 rows from the item's first
+// row on: a decoded token's heads, or 16 rows of a short portion (sequences with many rows go to the kernel
+// further down that shares keys and values through LDS).  Wavefront w takes the item's tiles of 32 keys
+// w, w + 4, ... (so that the block reads consecutive memory), and the four combine their results through
+// LDS at the end: four times the loads in flight for the same number of partial results, and a key range
+// of up to 2,048 keys leaves no partial results at all.  Which wavefront takes which tile follows from the
+// item alone, so a row's result still does not depend on the rest of the batch.
+//
+// A wavefront has its tile's values and the next tile's keys in flight while it computes; the loads of the
+// next tile's keys stand in straight-line code (the last tile is processed apart), since a branch around them
+// makes the compiler wait for every load in flight where the paths meet.  (Keys and values both a whole tile
+// ahead, in two sets of registers, need more than 256 registers and spill.)
+// PAGE32 (pages of a multiple of 32 keys): a tile lies in one page, whose number is read as a
+// scalar; the scalar loads count apart from the vector loads, so looking up the next page does not wait for
+// the loads in flight (a lookup by vector load, which returns in order behind them, would).  The values are
+// read in whole cache lines, once: their loads are non-temporal and leave the caches alone (1,074 MB of a
+// global layer at batch 8 and 32,768 tokens: 196 us before, 178 us with this alone).
+#define TEAM 4
+typedef const __attribute__((address_space(4))) int* scalar_ints;  // constant address space: a uniform index is read by a scalar load
+
+template <bool PAGE32>
 __global__ void __launch_bounds__(256, 2)
 attention_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long out_stride,
                       const bf16_t* __restrict__ cache, const int* __restrict__ block_table, int table_width,
@@ -136,11 +151,11 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __res
                       int n_work, float* __restrict__ partial, int n_q_heads, int n_kv_heads, int page_size,
                       int page_shift, int num_pages, int window_left, float scale_log2e) {
   const int lane = threadIdx.x & 63;
-  const int wave = UNIFORM_WAVE ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : (int)(threadIdx.x >> 6);
-  const long long id = (long long)blockIdx.x * (blockDim.x >> 6) + wave;
-  if (id >= (long long)n_work * n_kv_heads) return;
-  const int item = (int)(id / n_kv_heads);
-  const int g = (int)(id - (long long)item * n_kv_heads);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int id = blockIdx.x;  // (item, key/value head): the same for the whole block
+  const int item = id / n_kv_heads;
+  const int g = id - item * n_kv_heads;
+  if (item >= n_work) return;
   const int* w = work + (size_t)item * WORK_INTS;
   const int b = w[0];
   const int row0 = w[1];
@@ -158,76 +173,54 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __res
   const int n = lane & 15;  // row of the tile (B operands, results), key or dim of the tile (A operands)
   const int j = lane >> 4;
 
-  // this lane's rows, one per tile
-  bool row_valid[RT];
-  int ti[RT], hq[RT], row_end[RT], row_start[RT];
-  int lo_any = 0x7fffffff, hi_any = -1;
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    const int r = row0 + 16 * rt + n;
-    row_valid[rt] = r < n_rows;
-    ti[rt] = row_valid[rt] ? r / group : 0;
-    hq[rt] = g * group + (row_valid[rt] ? r - ti[rt] * group : 0);
-    row_end[rt] = n_old + ti[rt];  // last key the row may read
-    row_start[rt] = window_left >= 0 ? max(0, row_end[rt] - window_left) : 0;
-    if (row_valid[rt]) {
-      lo_any = min(lo_any, row_start[rt]);
-      hi_any = max(hi_any, row_end[rt]);
-    }
-  }
-  // the span of keys that any row of the wavefront reads (wave-uniform): outside it values
-  // may be anything (pages given back, slots never written) and are zeroed before use
+  // this lane's row
+  const int r = row0 + n;
+  const bool row_valid = r < n_rows;
+  const int ti = row_valid ? r / group : 0;
+  const int hq = g * group + (row_valid ? r - ti * group : 0);
+  const int row_end = n_old + ti;  // last key the row may read
+  const int row_start = window_left >= 0 ? max(0, row_end - window_left) : 0;
+  // the span of keys that any row of the item reads (uniform): outside it values may be anything
+  // (pages given back, slots never written) and are zeroed before use
+  int lo_any = row_valid ? row_start : 0x7fffffff, hi_any = row_valid ? row_end : -1;
+  // a tile every key of which every row reads needs no masks: from the latest first key to
+  // the earliest last key over the rows (never, if some row of the tile does not exist)
+  int lo_all = max(key_begin, row_valid ? row_start : 0x7fffffff), hi_all = min(key_end - 1, row_valid ? row_end : -1);
 #pragma unroll
   for (int off = 1; off < 16; off <<= 1) {
     lo_any = min(lo_any, __shfl_xor(lo_any, off, 64));
     hi_any = max(hi_any, __shfl_xor(hi_any, off, 64));
-  }
-  lo_any = max(lo_any, key_begin);
-  hi_any = min(hi_any, key_end - 1);
-  // a tile every key of which every row reads needs no masks: from the latest first key to
-  // the earliest last key over the rows (never, if some row of a tile does not exist)
-  int lo_all = key_begin, hi_all = key_end - 1;
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    lo_all = max(lo_all, row_valid[rt] ? row_start[rt] : 0x7fffffff);
-    hi_all = min(hi_all, row_valid[rt] ? row_end[rt] : -1);
-  }
-#pragma unroll
-  for (int off = 1; off < 16; off <<= 1) {
     lo_all = max(lo_all, __shfl_xor(lo_all, off, 64));
     hi_all = min(hi_all, __shfl_xor(hi_all, off, 64));
   }
+  lo_any = max(lo_any, key_begin);
+  hi_any = min(hi_any, key_end - 1);
 
   // queries: B operand, kept in registers for the whole loop
-  Frag8 qf[RT][K32_STEPS];
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    const bf16_t* qrow = q + (size_t)(q0 + ti[rt]) * q_stride + (size_t)hq[rt] * HEAD_DIM;
+  Frag8 qf[K32_STEPS];
+  {
+    const bf16_t* qrow = q + (size_t)(q0 + ti) * q_stride + (size_t)hq * HEAD_DIM;
 #pragma unroll
     for (int s = 0; s < K32_STEPS; ++s) {
       const bool filled = !(HALF_LAST_STEP && s == K32_STEPS - 1) || j < 2;
-      if (row_valid[rt] && filled)
-        qf[rt][s].u = *(const uint4*)(qrow + 32 * s + 8 * j);
+      if (row_valid && filled)
+        qf[s].u = *(const uint4*)(qrow + 32 * s + 8 * j);
       else
-        qf[rt][s].u = make_uint4(0, 0, 0, 0);
+        qf[s].u = make_uint4(0, 0, 0, 0);
     }
   }
 
-  float4v acc[RT][D_TILES];
-  float m_run[RT], neg_mc_run[RT], l_run[RT];  // l: this lane's share of the row's sum; the four lanes of a row are added at the end
+  float4v acc[D_TILES];
   const float neg_inf = -__builtin_inff();
   const float lazy_raw = 8.0f / scale_log2e;  // 8 binary orders, in units of the raw scores
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-#pragma unroll
-    for (int dt = 0; dt < D_TILES; ++dt) acc[rt][dt] = (float4v){0.f, 0.f, 0.f, 0.f};
-    m_run[rt] = neg_inf;
-    neg_mc_run[rt] = 0.f;
-    l_run[rt] = 0.f;
-  }
+  for (int dt = 0; dt < D_TILES; ++dt) acc[dt] = (float4v){0.f, 0.f, 0.f, 0.f};
+  float m_run = neg_inf, neg_mc_run = 0.f;
+  float l_run = 0.f;  // this lane's share of the row's sum; the four lanes of a row are added at the end
 
   const size_t plane = (size_t)n_kv_heads * page_size * HEAD_DIM;
   const int* table = block_table + (size_t)b * table_width;
+  const scalar_ints table_s = (scalar_ints)table;
   const bf16_t* kbase = cache + (size_t)g * page_size * HEAD_DIM;
   const bf16_t* vbase = cache + plane + (size_t)g * page_size * HEAD_DIM;
   // a key that some row reads must have a page: if its table entry is -1 or out of range the rows'
@@ -244,73 +237,60 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __res
   // keys of the two 16-key tiles that this lane loads rows of: 8*(n/4) + 4*t + n%4
   const int krel0 = 8 * (n >> 2) + (n & 3);
 
-  const int kt_first = key_begin & ~31;
-  Frag8 kf[2][K32_STEPS];
-  int vslot;
-  int vpage;
-  {
-    int ks0, ks1;
-    const int p0 = page_of(kt_first + krel0, ks0);
-    const int p1 = page_of(kt_first + krel0 + 4, ks1);
+  // page and first slot of the tile of 32 keys from `kt` on, for the lane's two key rows and its values
+  auto locate = [&](int kt, int& p0, int& ks0, int& p1, int& ks1, int& vp, int& vs) {
+    if (PAGE32) {
+      const int lp = page_shift >= 0 ? (kt >> page_shift) : (kt / page_size);  // uniform
+      const int first = kt - lp * page_size;
+      int page = lp < table_width ? table_s[lp] : 0;
+      page = (page >= 0 && page < num_pages) ? page : 0;
+      p0 = p1 = vp = page;
+      ks0 = first + krel0;
+      ks1 = ks0 + 4;
+      vs = first + 8 * j;
+    } else {
+      p0 = page_of(kt + krel0, ks0);
+      p1 = page_of(kt + krel0 + 4, ks1);
+      vp = page_of(kt + 8 * j, vs);
+    }
+  };
+  // the loads of that tile's keys (A operands, two tiles of 16 keys) ...
+  auto issue_keys = [&](Frag8 (&KF)[2][K32_STEPS], int kt) {
+    int ks0, ks1, vs, p0, p1, vp;
+    locate(kt, p0, ks0, p1, ks1, vp, vs);
     const bf16_t* kr0 = kbase + (size_t)p0 * 2 * plane + (size_t)ks0 * HEAD_DIM;
     const bf16_t* kr1 = kbase + (size_t)p1 * 2 * plane + (size_t)ks1 * HEAD_DIM;
 #pragma unroll
     for (int s = 0; s < K32_STEPS; ++s) {
       const bool filled = !(HALF_LAST_STEP && s == K32_STEPS - 1) || j < 2;
-      kf[0][s].u = filled ? *(const uint4*)(kr0 + 32 * s + 8 * j) : make_uint4(0, 0, 0, 0);
-      kf[1][s].u = filled ? *(const uint4*)(kr1 + 32 * s + 8 * j) : make_uint4(0, 0, 0, 0);
+      KF[0][s].u = filled ? *(const uint4*)(kr0 + 32 * s + 8 * j) : make_uint4(0, 0, 0, 0);
+      KF[1][s].u = filled ? *(const uint4*)(kr1 + 32 * s + 8 * j) : make_uint4(0, 0, 0, 0);
     }
-    vpage = page_of(kt_first + 8 * j, vslot);
-  }
-
-  for (int kt = kt_first; kt < key_end; kt += 32) {
-    const int nkt = kt + 32;
-    const bool has_next = nkt < key_end;
-
-    // ---- this tile's values: in flight while the scores are computed ------------------ //
-    // values of a page are stored in blocks of 8 keys, [slot / 8][dim][slot % 8]: the lane's
-    // 8 keys of one dimension are 16 contiguous bytes and 16 lanes read 256 contiguous bytes
-    Frag8 vf[D_TILES];
-    {
-      const bf16_t* vrow = vbase + (size_t)vpage * 2 * plane + ((size_t)(vslot >> 3) * HEAD_DIM + n) * 8;
+  };
+  // ... and of its values: stored in blocks of 8 keys, [slot / 8][dim][slot % 8], so the lane's 8 keys of one
+  // dimension are 16 contiguous bytes and 16 lanes read 256 contiguous bytes
+  auto issue_values = [&](Frag8 (&VF)[D_TILES], int kt) {
+    int ks0, ks1, vs, p0, p1, vp;
+    locate(kt, p0, ks0, p1, ks1, vp, vs);
+    const bf16_t* vrow = vbase + (size_t)vp * 2 * plane + ((size_t)(vs >> 3) * HEAD_DIM + n) * 8;
 #pragma unroll
-      for (int dt = 0; dt < D_TILES; ++dt) vf[dt].u = *(const uint4*)(vrow + dt * 16 * 8);
+    for (int dt = 0; dt < D_TILES; ++dt) VF[dt].w = __builtin_nontemporal_load((const u32x4*)(vrow + dt * 16 * 8));
+  };
+
+  // S^T = K Q^T for the 32 keys of a tile
+  auto scores = [&](Frag8 (&KF)[2][K32_STEPS], float4v (&st)[2]) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      float4v s_acc = (float4v){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < K32_STEPS; ++s) s_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(KF[t][s].v, qf[s].v, s_acc, 0, 0, 0);
+      st[t] = s_acc;
     }
-    // ---- pages of the next tile --------------------------------------------------------- //
-    int nks0 = 0, nks1 = 0, nvs = 0, np0 = 0, np1 = 0, nvp = 0;
-    if (has_next) {
-      np0 = page_of(nkt + krel0, nks0);
-      np1 = page_of(nkt + krel0 + 4, nks1);
-      nvp = page_of(nkt + 8 * j, nvs);
-    }
-
-    // ---- S^T = K Q^T for 32 keys, every row tile ------------------------------------------ //
-    float4v st[RT][2];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        float4v s_acc = (float4v){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < K32_STEPS; ++s)
-          s_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][s].v, qf[rt][s].v, s_acc, 0, 0, 0);
-        st[rt][t] = s_acc;
-      }
-
-    // ---- the next tile's keys: in flight during the softmax and the value product -------- //
-    if (has_next) {
-      const bf16_t* kr0 = kbase + (size_t)np0 * 2 * plane + (size_t)nks0 * HEAD_DIM;
-      const bf16_t* kr1 = kbase + (size_t)np1 * 2 * plane + (size_t)nks1 * HEAD_DIM;
-#pragma unroll
-      for (int s = 0; s < K32_STEPS; ++s) {
-        const bool filled = !(HALF_LAST_STEP && s == K32_STEPS - 1) || j < 2;
-        kf[0][s].u = filled ? *(const uint4*)(kr0 + 32 * s + 8 * j) : make_uint4(0, 0, 0, 0);
-        kf[1][s].u = filled ? *(const uint4*)(kr1 + 32 * s + 8 * j) : make_uint4(0, 0, 0, 0);
-      }
-    }
-
+  };
+  // masks, softmax and the value product of the tile from `kt` on
+  auto finish = [&](float4v (&st)[2], Frag8 (&VF)[D_TILES], int kt) {
     const bool need_mask = kt < lo_all || kt + 31 > hi_all;
-    // ---- values outside the span that any row reads are zeroed ---------------------------- //
+    // ---- values outside the span that any row reads are zeroed ---------------------------------- //
     const int vkey = kt + 8 * j;
     const bool boundary = (kt < lo_any) || (kt + 31 > hi_any);
     if (boundary) {
@@ -322,71 +302,97 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __res
       }
 #pragma unroll
       for (int dt = 0; dt < D_TILES; ++dt) {
-        vf[dt].u.x &= keep[0];
-        vf[dt].u.y &= keep[1];
-        vf[dt].u.z &= keep[2];
-        vf[dt].u.w &= keep[3];
+        VF[dt].u.x &= keep[0];
+        VF[dt].u.y &= keep[1];
+        VF[dt].u.z &= keep[2];
+        VF[dt].u.w &= keep[3];
       }
     }
-
+    // ---- mask, running maximum, probabilities --------------------------------------------------- //
+    float alpha;
+    Frag8 pf;
+    SOFTMAX_TILE(false, st[0], st[1], need_mask, row_valid && key >= row_start && key <= row_end && key >= key_begin && key < key_end,
+                 m_run, neg_mc_run, l_run, alpha, pf)
+    if (__any(alpha != 1.0f)) {  // seldom after the first tiles
+      asm volatile("" ::: "memory");  // keeps this a branch: unconditional, it is 4 multiplications per output tile
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      // ---- mask, running maximum, probabilities ------------------------------------------------ //
-      float alpha;
-      Frag8 pf;
-      SOFTMAX_TILE(false, st[rt][0], st[rt][1], need_mask,
-                   row_valid[rt] && key >= row_start[rt] && key <= row_end[rt] && key >= key_begin && key < key_end,
-                   m_run[rt], neg_mc_run[rt], l_run[rt], alpha, pf)
-      if (__any(alpha != 1.0f)) {  // seldom after the first tiles
-        asm volatile("" ::: "memory");  // keeps this a branch: unconditional, it is 4 multiplications per output tile
-#pragma unroll
-        for (int dt = 0; dt < D_TILES; ++dt) {
-          acc[rt][dt][0] *= alpha;
-          acc[rt][dt][1] *= alpha;
-          acc[rt][dt][2] *= alpha;
-          acc[rt][dt][3] *= alpha;
-        }
-      }
-
-      // ---- O^T += V^T P^T ------------------------------------------------------------------- //
-#pragma unroll
-      for (int dt = 0; dt < D_TILES; ++dt) {
-        acc[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf.v, acc[rt][dt], 0, 0, 0);
-      }
+      for (int dt = 0; dt < D_TILES; ++dt) acc[dt] *= alpha;
     }
-    vpage = nvp;
-    vslot = nvs;
+    // ---- O^T += V^T P^T ------------------------------------------------------------------------- //
+#pragma unroll
+    for (int dt = 0; dt < D_TILES; ++dt) acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(VF[dt].v, pf.v, acc[dt], 0, 0, 0);
+  };
+
+  // wavefront w starts at the item's tile w and goes on in steps of TEAM tiles
+  const int kt_step = 32 * TEAM;
+  const int kt_first = (key_begin & ~31) + 32 * wave;
+  Frag8 kf[2][K32_STEPS], vf[D_TILES];
+  if (kt_first < key_end) {
+    issue_keys(kf, kt_first);
+    int kt = kt_first;
+    for (; kt + kt_step < key_end; kt += kt_step) {
+      float4v st[2];
+      issue_values(vf, kt);
+      scores(kf, st);
+      issue_keys(kf, kt + kt_step);  // the next tile's keys: in flight during the softmax and the value product
+      finish(st, vf, kt);
+    }
+    float4v st[2];
+    issue_values(vf, kt);
+    scores(kf, st);
+    finish(st, vf, kt);
   }
 
+  // ---- the team's wavefronts combine: the largest reference maximum, every wavefront's sums and output
+  // scaled to it, and each wavefront adds up and stores a share of the dimensions ------------------------ //
+  __shared__ float team_m[TEAM][16], team_l[TEAM][16];
+  __shared__ __attribute__((aligned(16))) float team_o[TEAM][16][HEAD_DIM + 4];
+  float l_row = l_run;
+  l_row += __shfl_xor(l_row, 16, 64);
+  l_row += __shfl_xor(l_row, 32, 64);
+  if (j == 0) {
+    team_m[wave][n] = m_run;
+    team_l[wave][n] = l_row;
+  }
+  __syncthreads();
+  float m_all = neg_inf;
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    float l_row = l_run[rt];
-    l_row += __shfl_xor(l_row, 16, 64);
-    l_row += __shfl_xor(l_row, 32, 64);
-    if (!row_valid[rt]) continue;
+  for (int w2 = 0; w2 < TEAM; ++w2) m_all = fmaxf(m_all, team_m[w2][n]);
+  float l_all = 0.f, mine = 0.f;
+#pragma unroll
+  for (int w2 = 0; w2 < TEAM; ++w2) {
+    const float mw = team_m[w2][n];  // -inf: that wavefront had no tile, or none with a key of this row
+    const float f = (mw == neg_inf) ? 0.f : __builtin_amdgcn_exp2f((mw - m_all) * scale_log2e);
+    l_all += team_l[w2][n] * f;
+    if (w2 == wave) mine = f;
+  }
+#pragma unroll
+  for (int dt = 0; dt < D_TILES; ++dt) *(float4v*)&team_o[wave][n][16 * dt + 4 * j] = acc[dt] * mine;
+  __syncthreads();
+  if (!row_valid) return;
+  const float inv = page_missing ? not_a_number() : 1.0f / l_all;
+  bf16_t* orow = out + (size_t)(q0 + ti) * out_stride + (size_t)hq * HEAD_DIM;
+  float* prow = slot < 0 ? nullptr : partial + (((size_t)slot * n_kv_heads + g) * 16 + n) * PARTIAL_STRIDE;
+  for (int dt = wave; dt < D_TILES; dt += TEAM) {
+    float4v sum = *(const float4v*)&team_o[0][n][16 * dt + 4 * j];
+#pragma unroll
+    for (int w2 = 1; w2 < TEAM; ++w2) sum += *(const float4v*)&team_o[w2][n][16 * dt + 4 * j];
     if (slot < 0) {
-      // the whole key range was this wavefront's: normalise and store
-      const float inv = page_missing ? not_a_number() : 1.0f / l_row;
-      bf16_t* orow = out + (size_t)(q0 + ti[rt]) * out_stride + (size_t)hq[rt] * HEAD_DIM;
-#pragma unroll
-      for (int dt = 0; dt < D_TILES; ++dt) {
-        uint2 v;
-        v.x = pack_bf16(acc[rt][dt][0] * inv, acc[rt][dt][1] * inv);
-        v.y = pack_bf16(acc[rt][dt][2] * inv, acc[rt][dt][3] * inv);
-        *(uint2*)(orow + 16 * dt + 4 * j) = v;
-      }
+      // the whole key range was this block's: normalise and store
+      uint2 v;
+      v.x = pack_bf16(sum[0] * inv, sum[1] * inv);
+      v.y = pack_bf16(sum[2] * inv, sum[3] * inv);
+      *(uint2*)(orow + 16 * dt + 4 * j) = v;
     } else {
-      // (split items have one row tile)
-      float* prow = partial + (((size_t)slot * n_kv_heads + g) * 16 + n) * PARTIAL_STRIDE;
-#pragma unroll
-      for (int dt = 0; dt < D_TILES; ++dt) *(float4v*)(prow + 16 * dt + 4 * j) = acc[rt][dt];
-      if (j == 0) {
-        prow[HEAD_DIM] = m_run[rt] * scale_log2e;  // the merge works in the scaled (log2) domain
-        prow[HEAD_DIM + 1] = page_missing ? not_a_number() : l_row;  // the merged row becomes NaN too
-      }
+      *(float4v*)(prow + 16 * dt + 4 * j) = sum;
     }
+  }
+  if (slot >= 0 && wave == 0 && j == 0) {
+    prow[HEAD_DIM] = m_all * scale_log2e;  // the merge works in the scaled (log2) domain
+    prow[HEAD_DIM + 1] = page_missing ? not_a_number() : l_all;  // the merged row becomes NaN too
   }
 }
+#undef TEAM
 
 // ---- prompt portions: 64 * LDS_RT rows per block, keys and values shared through LDS ------- //
 // work item: {sequence, first row, first key, end key (exclusive), partial slot or -1, chunks of
@@ -994,22 +1000,20 @@ extern "C" int cwm_attention_mfma(const void* q, long q_stride, void* out, long 
   }
   int status = 0;
   if (n_work > 0) {
-    // few wavefronts: one per block, so that they spread over all compute units; many: four per block
-    const long long waves = (long long)n_work * n_kv_heads;
-    const int per_block = waves <= 6144 ? 1 : 4;
-    const long long blocks = (waves + per_block - 1) / per_block;
+    // a block of four wavefronts per (item, key/value head)
+    const long long blocks = (long long)n_work * n_kv_heads;
     CWM_REQUIRE(blocks <= 0x7fffffffLL, "attention_mfma: too many work items");
-    // work_keys: the keys of an average item
-#define CWM_LAUNCH_SPLIT(UNIFORM)                                                                                       \
-  hipLaunchKernelGGL((attention_mfma_kernel<1, UNIFORM>), dim3((unsigned)blocks), dim3(64 * per_block), 0, stream,        \
-                     (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)cache, block_table, table_width, \
-                     cu_q, kv_len, work, n_work, partial, n_q_heads, n_kv_heads, page_size, page_shift, num_pages,       \
-                     window_left, scale_log2e)
-    if (work_keys < 192)
-      CWM_LAUNCH_SPLIT(true);
+    (void)work_keys;
+#define CWM_LAUNCH_TEAM(PAGE32)                                                                                          \
+  hipLaunchKernelGGL((attention_mfma_kernel<PAGE32>), dim3((unsigned)blocks), dim3(256), 0, stream, (const bf16_t*)q,     \
+                     q_stride, (bf16_t*)out, out_stride, (const bf16_t*)cache, block_table, table_width, cu_q, kv_len,   \
+                     work, n_work, partial, n_q_heads, n_kv_heads, page_size, page_shift, num_pages, window_left,        \
+                     scale_log2e)
+    if (page_size % 32 == 0)
+      CWM_LAUNCH_TEAM(true);
     else
-      CWM_LAUNCH_SPLIT(false);
-#undef CWM_LAUNCH_SPLIT
+      CWM_LAUNCH_TEAM(false);
+#undef CWM_LAUNCH_TEAM
     status = cwm_launch_status("attention_mfma");
     if (status) return status;
   }

@@ -2,8 +2,8 @@
 
 For every sequence and 16-row tile (rows are (token, head of the group) pairs) the
 list names the keys the tile reads.  A sequence that brings few rows (a decoded
-token, a short portion) has its key range cut into chunks at fixed absolute
-positions so that many wavefronts share the reading; the chunks' partial results
+token, a short portion) has a long key range cut into chunks at fixed absolute
+positions so that many blocks share the reading; the chunks' partial results
 are merged by a second kernel.  Whether and where a sequence is cut depends on its
 own lengths only.
 """
@@ -23,13 +23,15 @@ WIDE_CHUNK_FINE = 2048  # the same for a sequence with very few such blocks
 
 
 def chunk_keys(n_keys):
-    """Keys per chunk (a multiple of 32) for a tile that reads `n_keys` keys (a number or
-    an array of them): short ranges are cut finer so that a lone decoded token still
-    spreads over the chip; long ones coarser, since every chunk costs a wavefront's start
-    and a partial result to merge.  (Measured at batch 1, 8 and 64: a batch of 8 or more
-    would take 512 keys from 5,000 on, a lone sequence 128 up to 12,000.)"""
+    """Keys per chunk (a multiple of 128: four wavefronts take a chunk's tiles of 32 keys in turn) for a row tile
+    that reads `n_keys` keys (a number or an array of them).  Up to 2,048 keys are not cut: a block of four
+    wavefronts reads them and leaves no partial result (64 sequences of 1,024 keys: 45 us a layer of the 32B
+    shape against 59 us in two chunks with their merge; a lone sequence of 1,024 keys pays 15 us against 10 us
+    in chunks of 256).  Longer ranges are cut so that a few sequences still spread over the chip: 512 keys up
+    to 8,192 (eight sequences in a window of 8,192 keys: 54 us against 58 us in chunks of 1,024), 1,024 up to
+    65,536, then 2,048 (eight sequences of 131,072 keys: 647 us against 665 us in chunks of 4,096)."""
     n = np.asarray(n_keys)
-    return np.where(n <= 2048, 64, np.where(n <= 4096, 128, np.where(n <= 8192, 256, np.where(n <= 65536, 512, 1024))))
+    return np.where(n <= 2048, 2048, np.where(n <= 8192, 512, np.where(n <= 65536, 1024, 2048)))
 
 
 MERGE_MID_MAX = 32  # partials up to which an item is merged by 4 wavefronts instead of 16

@@ -614,8 +614,9 @@ def test_attention_mfma(n_q, n_kv, hd, page_size, window):
 
 @pytest.mark.parametrize("window", [None, 20000])
 def test_attention_mfma_long_ranges(window):
-    """Decoded tokens and short portions far into long sequences: every chunk length of the
-    split (64, 128, 256, 512 and 1,024 keys) and the merge of up to 69 partial results, against
+    """Decoded tokens and short portions far into long sequences: uncut ranges of up to 2,048 keys (four
+    wavefronts of a block combine), every chunk length of the split (512, 1,024 and 2,048 keys) and the
+    merge of up to 35 partial results, against
     float32 torch on the device.  One far key stands out in the longest sequence.  The last two
     sequences bring portions of many rows but too few blocks for the chip: their blocks' keys
     are cut (at multiples of 2,048 and of 8,192) and merged as well."""
@@ -678,8 +679,8 @@ def test_attention_mfma_long_ranges(window):
 @pytest.mark.parametrize("window", [None, 8192])
 def test_attention_mfma_long_ranges_with_heads_of_128_and_pages_of_256(window):
     """The geometry of a long-context decode step of the 32B shape (48 query heads on 8 key/value heads
-    of 128, pages of 256 keys): decoded tokens after 32,767 and 131,071 keys (chunks of 512 and 1,024 keys,
-    up to 128 partial results a row) and a portion of three rows after 100,000, against float32 torch on
+    of 128, pages of 256 keys): decoded tokens after 32,767 and 131,071 keys (chunks of 1,024 and 2,048 keys,
+    up to 64 partial results a row) and a portion of three rows after 100,000, against float32 torch on
     the device.  Everything is made on the device; one far key stands out for the longest sequence."""
     from types import SimpleNamespace
 
