@@ -108,6 +108,11 @@ __device__ __forceinline__ void dma16(const bf16_t* base, uint32_t offset, uint3
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(offset), "s"(base) : "memory", "m0");
 }
 
+// The same past the caches (non-temporal): for data that is read once, in whole cache lines per instruction.
+__device__ __forceinline__ void dma16_once(const bf16_t* base, uint32_t offset, uint32_t lds) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" : : "s"(lds), "v"(offset), "s"(base) : "memory", "m0");
+}
+
 // ---- host side: error channel ------------------------------------------------ //
 static thread_local char cwm_error_buffer[512] = {0};
 

@@ -137,7 +137,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restric
     const bf16_t* as = asrc + (size_t)k_step * TL_BK;
     const uint32_t dst = lds0 + buf * STAGE;
 #pragma unroll
-    for (int i = 0; i < W_DMA; ++i) dma16(ws, w_off[i], dst + (wave * W_DMA + i) * 1024);
+    for (int i = 0; i < W_DMA; ++i) dma16_once(ws, w_off[i], dst + (wave * W_DMA + i) * 1024);  // W is read once, 8 rows of 128 bytes a load
 #pragma unroll
     for (int i = 0; i < A_DMA; ++i) dma16(as, a_off[i], dst + W_BYTES + (wave * A_DMA + i) * 1024);
     if (i_left > 1) {  // past the block's last pair: that pair again, into a buffer nobody reads
