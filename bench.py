@@ -296,6 +296,8 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=32768)
     ap.add_argument("--page", type=int, default=256)
     ap.add_argument("--no-points", action="store_true")
+    ap.add_argument("--prefill-tokens", type=int, default=2048, help="tokens of the prompt portion that `prefill` times")
+    ap.add_argument("--prefill-offset", type=int, default=0, help="tokens already cached before that portion (0: a fresh prompt)")
     ap.add_argument("--no-ceilings", action="store_true", help="do not measure what the GPU reaches (the read rate and the matrix instruction's rate)")
     ap.add_argument("--graphs", type=int, default=16, help="decode steps kept as HIP graphs where the host is the limit, as the engine's default (0: none)")
     ap.add_argument(
@@ -343,15 +345,17 @@ def main() -> int:
         roofline["peak_measured_100mb"] = ceilings["read_100mb"]
         roofline["peak_measured_500mb"] = ceilings["read_500mb"]
 
-    n_prefill = 2048
-    prefill_s = bench.prefill_run(n_prefill)
-    prefill_rate = bench.prefill_flops(n_prefill) / prefill_s
+    n_prefill = args.prefill_tokens
+    prefill_s = bench.prefill_run(n_prefill, offset=args.prefill_offset)
+    prefill_rate = bench.prefill_flops(n_prefill, offset=args.prefill_offset) / prefill_s
     prefill = {
         "value": round(n_prefill / prefill_s, 1),
         "tokens": n_prefill,
         "ms": round(prefill_s * 1e3, 2),
         "frac": round(prefill_rate / PEAK_FLOPS[args.dtype], 4),
     }
+    if args.prefill_offset:
+        prefill["offset"] = args.prefill_offset
     if ceilings and args.dtype == "bf16":
         prefill["peak_measured"] = ceilings["mfma_bf16"]  # TFLOP/s of the matrix instruction issued from registers
         prefill["frac_measured"] = round(prefill_rate / (ceilings["mfma_bf16"] * 1e12), 4)
@@ -392,9 +396,9 @@ def main() -> int:
         tok_s_70, ms_70 = other.decode_run(8, 8192, 20, 4)
         points["llama70b_decode_b8"] = round(tok_s_70, 1)
         points["llama70b_decode_b8_frac"] = hbm_fractions(other.step_bytes(8, 8192), ms_70)[1]
-        seconds = other.prefill_run(n_prefill)
-        points["llama70b_prefill"] = round(n_prefill / seconds, 1)
-        points["llama70b_prefill_frac"] = round(other.prefill_flops(n_prefill) / seconds / PEAK_FLOPS[args.dtype], 4)
+        seconds = other.prefill_run(2048)
+        points["llama70b_prefill"] = round(2048 / seconds, 1)
+        points["llama70b_prefill_frac"] = round(other.prefill_flops(2048) / seconds / PEAK_FLOPS[args.dtype], 4)
         other.close()
 
     line = {

@@ -192,7 +192,7 @@ def gate_up_silu(
         and x.shape[0] <= STREAM_EPILOGUE_ROWS and _stream_takes(x, weight)
         and x.shape[1] <= stream_unsplit_k(x.shape[0])  # K fits one group of wavefronts: no split
     )
-    tiled = x.is_cuda and x.dim() == 2 and _prefers_tile(x, weight, bias)
+    tiled = x.is_cuda and x.dim() == 2 and _prefers_tile(x, weight, bias, streamed)
     if fused and not tiled:
         return gemm_bf16_stream(x, weight, bias, torch.bfloat16, glu=True, streamed=streamed)
     if tiled and grouped and x.shape[0] <= TILE_ROWS:
@@ -485,7 +485,7 @@ def qkv_rope_write(
         and head_dim <= 256
         and _stream_takes(x, weight)
         and x.shape[1] <= stream_unsplit_k(x.shape[0])  # K fits one group of wavefronts: no split
-        and not _prefers_tile(x, weight, bias)
+        and not _prefers_tile(x, weight, bias, streamed)
     )
     if fused:
         _i32(positions, "positions")
@@ -660,9 +660,21 @@ TILE_TALL_ROWS = 256  # rows of its tallest block: up to there it reads W once
 TILE_COLUMNS = 128  # columns of a tall block's tile
 
 
-def _prefers_tile(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> bool:
-    """Whether this product goes to the tiled kernel (which has no bias of its own)."""
-    return x.shape[0] > STREAM_FUSED_ROWS and bias is None and _tile_wins(x, weight)
+# entries of a matrix from which on reading it is what a product of few rows costs (below, a launch more or less counts as much)
+TILE_FEW_ROWS_ENTRIES = 1 << 24
+
+
+def _prefers_tile(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], streamed: Optional[torch.Tensor] = None) -> bool:
+    """Whether this product goes to the tiled kernel (which has no bias of its own): from 9 rows on; and for
+    fewer rows where the matrix is large and has no streaming copy, since the tiled kernel reads the row-major
+    matrix in whole cache lines past the caches, which the streaming kernel can only do with that copy (a
+    layer's four products of the 32B shape at 8 rows: 159 us tiled, 187 us streamed from the row-major
+    matrices, 159 us streamed from the copies; at 1 row 163, 178 and 154 us)."""
+    if bias is not None:
+        return False
+    if x.shape[0] <= STREAM_FUSED_ROWS and (streamed is not None or weight.numel() < TILE_FEW_ROWS_ENTRIES):
+        return False
+    return _tile_wins(x, weight)
 
 
 def _tile_wins(x: torch.Tensor, weight: torch.Tensor) -> bool:
@@ -715,7 +727,7 @@ def gemm_bf16(
     m = x.shape[0]
     if not _stream_takes(x, weight):
         return gemm_f32(x, weight, bias, out_dtype)
-    if _prefers_tile(x, weight, bias):
+    if _prefers_tile(x, weight, bias, streamed):
         return gemm_bf16_tile(x, weight, None, out_dtype, partials_ok)
     if m <= STREAM_MAX_ROWS:
         return gemm_bf16_stream(x, weight, bias, out_dtype, partials_ok, streamed=streamed)

@@ -1234,6 +1234,31 @@ def test_products_of_9_to_128_rows_take_the_tiled_kernel():
     assert torch.equal(ops.gate_up_silu(xo[:12].contiguous(), odd, None, True), ops.gemm_bf16_stream(xo[:12].contiguous(), odd, None, torch.bfloat16, glu=True))
 
 
+def test_few_rows_of_a_large_matrix_take_the_tiled_kernel_unless_it_has_a_streaming_copy():
+    """Up to 8 rows: a large matrix (2**24 entries and more) without a streaming copy goes to the tiled kernel,
+    which reads the row-major matrix in whole cache lines past the caches; with the copy, and for small
+    matrices, the streaming kernel stays.  Each choice gives the bits of the kernel it names, and all of
+    them the right product."""
+    from cwm_amd import ops
+
+    x = rnd((5, 4096), torch.bfloat16, 31).to(DEV)
+    w = rnd((4096, 4096), torch.bfloat16, 32, 0.05).to(DEV)
+    assert w.numel() >= ops.TILE_FEW_ROWS_ENTRIES
+    want = x.double() @ w.double().T
+    tiled = ops.gemm_bf16_tile(x, w)
+    assert torch.equal(ops.linear(x, w), tiled)
+    copy = ops.stream_layout(w)
+    streamed = ops.gemm_bf16_stream(x, w, streamed=copy)
+    assert torch.equal(ops.linear(x, w, streamed=copy), streamed)
+    for got in (tiled, streamed):
+        torch.testing.assert_close(got.double(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+    # a gated product likewise: the tiled kernel's epilogue without the copy, the streaming kernel's with it
+    assert torch.equal(ops.gate_up_silu(x, w, None, True), ops.gemm_bf16_tile(x, w, glu=True))
+    assert torch.equal(ops.gate_up_silu(x, w, None, True, streamed=copy), ops.gemm_bf16_stream(x, w, None, torch.bfloat16, glu=True, streamed=copy))
+    small = w[:2048].contiguous()
+    assert torch.equal(ops.linear(x, small), ops.gemm_bf16_stream(x, small))
+
+
 @pytest.mark.parametrize("n_q,n_kv,hd,page_size,dim,m", [(4, 2, 16, 8, 64, 40), (6, 1, 64, 16, 128, 70), (12, 2, 128, 64, 256, 33), (3, 3, 48, 8, 192, 100)])
 def test_rope_kv_write_from_partial_sums(n_q, n_kv, hd, page_size, dim, m):
     """The q/k/v projection of 17 to 128 rows leaves partial sums; rotation and cache write take them
