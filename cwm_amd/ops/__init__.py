@@ -886,12 +886,13 @@ class StaticPlans:
         self.homes: dict = {}  # (group, key/value heads, window) -> (capacity, device vector, uploaded plan)
 
     def _padded(self, batch, group: int, n_kv: int, window: Optional[int], capacity):
-        from .attention_plan import PlanCapacity, build_plan, pad_plan
+        from .attention_plan import build_plan, capacity_until, pad_plan
 
         wide_cut_below = -(-2 * _compute_units(self.device) // n_kv)
-        plan = build_plan(batch.q_lens, batch.kv_lens, group, window, wide_cut_below)
         if capacity is None:
-            capacity = PlanCapacity.roomy(plan)
+            plan, capacity = capacity_until(batch.q_lens, batch.kv_lens, group, window, wide_cut_below, self.max_keys)
+        else:
+            plan = build_plan(batch.q_lens, batch.kv_lens, group, window, wide_cut_below)
         flat = pad_plan(plan, capacity)
         return plan, capacity, flat
 

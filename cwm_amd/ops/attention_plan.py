@@ -199,15 +199,43 @@ class PlanCapacity:
         return self.work * WORK_INTS + self.merge * 4
 
     @staticmethod
-    def roomy(plan: AttentionPlan) -> "PlanCapacity":
-        """Room for `plan` and for a quarter more keys: every tile's keys grow, so a tile that is not yet cut
-        will be, each gains a chunk now and then, and a merge item whose partials come near MERGE_MID_MAX will
-        move from the items of few partials to those of many (no item is near: no launch for those at all)."""
+    def covering(plans: Sequence[AttentionPlan]) -> "PlanCapacity":
+        """Room for the largest of `plans` in every list: the caller hands in the step's plan and the plans of the
+        same step with its sequences grown as far as the capture allows (and grown just to every length at which
+        the rule of `chunk_keys` changes, since a longer range may be cut into fewer chunks than a shorter one).  A
+        list that stays empty in all of them gets no launch at all."""
+        work = merge_many = merge_mid = 0
+        for plan in plans:
+            n_many = plan.merge.shape[0] - plan.n_merge_mid - plan.n_merge_wide
+            work = max(work, plan.work.shape[0])
+            merge_many = max(merge_many, n_many)
+            merge_mid = max(merge_mid, plan.n_merge_mid)
+        return PlanCapacity(work=work, merge_many=merge_many, merge_mid=merge_mid)
+
+
+# lengths of a key range at which `chunk_keys` changes (the last length of each rule)
+CHUNK_RULE_ENDS = (2048, 8192, 65536)
+
+
+def capacity_until(
+    q_lens: Sequence[int], kv_lens: Sequence[int], group: int, window: Optional[int], wide_cut_below: int, max_keys: int
+) -> "tuple[AttentionPlan, PlanCapacity]":
+    """The step's plan, and the sizes of its lists for as long as no sequence holds more than `max_keys` keys
+    (every sequence growing by a token a step): the sequences as they are, all of them grown to `max_keys`, and
+    grown to each length in between at which the rule for cutting the keys changes."""
+    plan = build_plan(q_lens, kv_lens, group, window, wide_cut_below)
+    plans = [plan]
+    for length in sorted({max_keys, *(n + d for n in CHUNK_RULE_ENDS for d in (0, 1) if n + d < max_keys)}):
+        grown = [min(max(kv, length), max(kv, max_keys)) for kv in kv_lens]
+        if grown != list(kv_lens):
+            plans.append(build_plan(q_lens, grown, group, window, wide_cut_below))
+    capacity = PlanCapacity.covering(plans)
+    if window is not None:
+        # a window's range moves over the fixed positions of the cuts: at some steps it straddles one cut more than at
+        # others, whatever its length (a window shorter than a chunk is cut in two now and then)
         tiles = int((plan.work[:, 4] < 0).sum()) + plan.merge.shape[0]
-        work = plan.work.shape[0]
-        near_many = int((plan.merge[:, 3] > (3 * MERGE_MID_MAX) // 4).sum())
-        many_now = plan.merge.shape[0] - plan.n_merge_mid - plan.n_merge_wide
-        return PlanCapacity(work=work + max(work // 4, 2 * tiles, 16), merge_many=near_many, merge_mid=tiles - many_now)
+        capacity = PlanCapacity(work=capacity.work + tiles, merge_many=capacity.merge_many, merge_mid=max(capacity.merge_mid, tiles))
+    return plan, capacity
 
 
 def pad_plan(plan: AttentionPlan, capacity: PlanCapacity) -> Optional[np.ndarray]:

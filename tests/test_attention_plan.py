@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 
 from cwm_amd.ops.attention_plan import (
+    capacity_until,
     MERGE_MID_MAX, NULL_ROW, ROWS_PER_TILE, WIDE_TILES, PlanCapacity, build_plan, pad_plan,
 )
 
@@ -81,8 +82,8 @@ def test_lists_of_a_fixed_length(seed):
     q, kv = random_batch(rng, decode_only=True)
     group = int(rng.choice([1, 4, 6, 16, 24]))
     window = None if rng.random() < 0.5 else int(rng.choice([8, 100, 8192]))
-    plan = build_plan(q, kv, group, window)
-    capacity = PlanCapacity.roomy(plan)
+    max_keys = int(max(kv) * rng.choice([1.0, 1.25, 1.6])) + int(rng.integers(1, 300))
+    plan, capacity = capacity_until(q, kv, group, window, 0, max_keys)
     flat = pad_plan(plan, capacity)
     assert flat is not None and flat.dtype == np.int32 and flat.size == capacity.ints
     work = flat[: capacity.work * 6].reshape(-1, 6)
@@ -96,12 +97,31 @@ def test_lists_of_a_fixed_length(seed):
     mid = merge[capacity.merge_many :]
     assert np.array_equal(mid[: plan.n_merge_mid], plan.merge[n_many:])
     assert (mid[plan.n_merge_mid :, 1] == NULL_ROW).all() and (mid[plan.n_merge_mid :, 3] == 0).all()
-    # the same requests some steps later still fit; much later they do not, and that is said
-    later = build_plan(q, [n + max(n // 8, 1) for n in kv], group, window)
-    assert pad_plan(later, capacity) is not None
-    much_later = build_plan(q, [4 * n + 5000 for n in kv], group, window)
+    # every later step of the same requests fits until the longest has `max_keys` keys: a token a step, checked at steps
+    # spread over the way and around every length at which the rule of the cut changes
+    room = max_keys - max(kv)
+    steps = set(np.linspace(0, room, 40).astype(int).tolist())
+    for n in kv:
+        for end in (2048, 8192, 65536):
+            steps |= {end - n + d for d in (-1, 0, 1, 2) if 0 <= end - n + d <= room}
+    for t in sorted(steps):
+        later = build_plan(q, [n + t for n in kv], group, window)
+        assert pad_plan(later, capacity) is not None, (t, kv, max_keys, window)
+    # much later they do not fit, and that is said
+    much_later = build_plan(q, [4 * n + 5000 + max_keys for n in kv], group, window)
     if window is None:
         assert pad_plan(much_later, capacity) is None
+
+
+def test_a_step_that_cannot_be_cut_has_no_merge_list():
+    """Sequences that stay within 2,048 keys while the capture is in use are never cut: the capture holds no
+    launch of the merge kernel at all.  One that may cross 2,048 keys has room for its partial results."""
+    _, capacity = capacity_until([1] * 5, [900, 1024, 1300, 40, 1700], 6, None, 0, 2040)
+    assert capacity.merge == 0 and capacity.work == 5
+    _, capacity = capacity_until([1] * 5, [900, 1024, 1300, 40, 1700], 6, None, 0, 2300)
+    assert capacity.merge_mid == 5 and capacity.work == 5 * 5  # 2,300 keys are five chunks of 512
+    _, capacity = capacity_until([1] * 2, [8000, 100], 6, None, 0, 10000)
+    assert capacity.work == 2 * 16  # 8,192 keys in 16 chunks of 512 are more items than 10,000 keys in 10 chunks of 1,024
 
 
 def test_a_step_with_blocks_of_many_rows_has_no_list_of_a_fixed_length():
