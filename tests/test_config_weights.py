@@ -271,3 +271,38 @@ def test_a_head_size_no_kernel_takes_is_refused_when_the_model_is_built():
     arch, cfg = parse_config(data)
     with pytest.raises(ValueError, match="head_dim 272"):
         Model(arch.build_plan(cfg))
+
+
+def test_streaming_copies_are_kept_where_the_matrices_fit_twice_into_half_the_memory(monkeypatch):
+    """The rule of `wants_stream_copies`: bfloat16 on a GPU only; an explicit choice or CWM_AMD_STREAM_COPIES
+    decides; else the matrices, twice, against half of the device's memory (32B shape: 127 GB of 288 fit,
+    70B shape: 278 GB do not)."""
+    import types
+
+    import torch
+
+    from cwm_amd.config import parse_config
+    from cwm_amd.engine import loading
+    from cwm_amd.models import Model
+
+    def model_of(**sizes):
+        config = {"architecture": "llama3_dense", "vocab_size": 128256, "ffn_dim_multiplier": 1.3, "multiple_of": 256, "head_dim": 128,
+                  "n_kv_heads": 8, "norm_eps": 1e-5, "rope_theta": 500000.0, **sizes}
+        arch, typed = parse_config(config)
+        return Model(arch.build_plan(typed))
+
+    small = model_of(dim=6144, n_layers=64, n_heads=48, ffn_dim_multiplier=1.3125)  # the 32B shape
+    large = model_of(dim=8192, n_layers=80, n_heads=64, multiple_of=4096)  # the 70B shape
+    gpu, cpu = torch.device("cuda:0"), torch.device("cpu")
+    monkeypatch.setattr(torch.cuda, "get_device_properties", lambda device: types.SimpleNamespace(total_memory=288 * 2**30))
+    monkeypatch.delenv("CWM_AMD_STREAM_COPIES", raising=False)
+    assert loading.wants_stream_copies(small, torch.bfloat16, gpu) is True
+    assert loading.wants_stream_copies(large, torch.bfloat16, gpu) is False
+    assert loading.wants_stream_copies(small, torch.float32, gpu) is False
+    assert loading.wants_stream_copies(small, torch.bfloat16, cpu) is False
+    assert loading.wants_stream_copies(large, torch.bfloat16, gpu, choice=True) is True
+    monkeypatch.setenv("CWM_AMD_STREAM_COPIES", "0")
+    assert loading.wants_stream_copies(small, torch.bfloat16, gpu) is False
+    assert loading.wants_stream_copies(small, torch.bfloat16, gpu, choice=True) is True  # the argument outranks the environment
+    monkeypatch.setenv("CWM_AMD_STREAM_COPIES", "1")
+    assert loading.wants_stream_copies(large, torch.bfloat16, gpu) is True

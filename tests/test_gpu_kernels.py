@@ -1377,3 +1377,20 @@ def test_attention_of_a_decoded_token_does_not_depend_on_the_batch(n_q, n_kv, hd
         assert torch.equal(run(list(range(start, start + 10))), together[start : start + 10]), f"sequences {start}.. differ"
     for b, w in want:
         torch.testing.assert_close(together[b].float(), w, rtol=2e-2, atol=2e-2)
+
+
+def test_ceiling_kernels_run_and_give_plausible_rates():
+    """The two kernels that say what the GPU reaches (not on the model's path): a read of 64 MB windows of a
+    256 MB buffer and a short loop of matrix instructions; sizes that the entry points do not take are refused."""
+    from cwm_amd import ops
+
+    buffer = torch.zeros(256 << 20, dtype=torch.uint8, device=DEV)
+    rate = ops.measure_read_rate(buffer, 64 << 20, 8, 2048)
+    assert 500.0 < rate < 20000.0, rate  # GB/s: far from nothing, not beyond any memory
+    with pytest.raises(ops.KernelError):
+        ops.measure_read_rate(buffer, (64 << 20) + 8, 2, 256)
+    for shape in (16, 32):
+        flops = ops.measure_mfma_rate(DEV, 512, 2000, launches=2, shape=shape)
+        assert 0.05 < flops < 5.0, flops  # PFLOP/s
+    with pytest.raises(ops.KernelError, match="shape"):
+        ops.measure_mfma_rate(DEV, 512, 10, shape=8)

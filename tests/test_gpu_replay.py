@@ -116,3 +116,40 @@ def test_many_requests_decode_together(folders, dtype):
     got = traces.gather(steps, outputs, {k: len(v) for k, v in requests.items()}, vocab)
     compare(got, cmp.expected(folders[name, dtype], requests, dtype), dtype, f"{name} {dtype} ninety requests")
     assert rep.manager.live_requests() == []
+
+
+@pytest.mark.parametrize("name", ["tiny_b", "tiny_d"])
+def test_streaming_copies_change_no_bit(folders, name):
+    """A model that keeps its matrices' streaming copies (the default where they fit) gives the logits of the same
+    model without them bit for bit, under a trace that mixes portions and single tokens: the copies hold the same
+    values, and the products add them in the same order."""
+    from cwm_amd.cache import CacheManager, CacheStorage
+    from cwm_amd.engine import ModelRunner, Portion, load_model
+
+    requests = requests_for(name)
+    steps = traces.mixed(requests)
+    outputs = {}
+    for copies in (False, True):
+        model, _ = load_model(folders[name, "bfloat16"], "bfloat16", "cuda:0", stream_copies=copies)
+        assert model.runtime.stream_copies == copies
+        assert (model.head.weights.streamed is not None) == copies
+        manager = CacheManager(model.cache_specs, 8, 2 * traces.max_live_tokens(steps) // 8, 8)
+        storage = CacheStorage(manager, model.runtime.device, model.runtime.act_dtype)
+        runner = ModelRunner(model, manager, storage)
+        got = []
+        for st in steps:
+            portions = []
+            for e in st["entries"]:
+                if not e["tokens"]:
+                    continue
+                if e["id"] not in manager:
+                    runner.admit(e["id"])
+                assert manager.extend(e["id"], len(e["tokens"]))
+                portions.append(Portion(e["id"], e["tokens"], e["want"]))
+            logits = runner.step(portions) if portions else None
+            if logits is not None:
+                got.append(logits.cpu())
+            for rid in st["end"]:
+                runner.release(rid)
+        outputs[copies] = torch.cat(got)
+    assert outputs[True].shape[0] > 100 and torch.equal(outputs[True], outputs[False])
