@@ -230,9 +230,10 @@ def capacity_until(
         if grown != list(kv_lens):
             plans.append(build_plan(q_lens, grown, group, window, wide_cut_below))
     capacity = PlanCapacity.covering(plans)
-    if window is not None:
+    if window is not None and max(max(kv_lens), max_keys) > window:
         # a window's range moves over the fixed positions of the cuts: at some steps it straddles one cut more than at
-        # others, whatever its length (a window shorter than a chunk is cut in two now and then)
+        # others, whatever its length (a window shorter than a chunk is cut in two now and then).  While no sequence
+        # is longer than the window every range starts at key 0, as without a window.
         tiles = int((plan.work[:, 4] < 0).sum()) + plan.merge.shape[0]
         capacity = PlanCapacity(work=capacity.work + tiles, merge_many=capacity.merge_many, merge_mid=max(capacity.merge_mid, tiles))
     return plan, capacity

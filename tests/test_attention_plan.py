@@ -118,6 +118,11 @@ def test_a_step_that_cannot_be_cut_has_no_merge_list():
     launch of the merge kernel at all.  One that may cross 2,048 keys has room for its partial results."""
     _, capacity = capacity_until([1] * 5, [900, 1024, 1300, 40, 1700], 6, None, 0, 2040)
     assert capacity.merge == 0 and capacity.work == 5
+    # the same in a layer whose window no sequence outgrows meanwhile; a window that one has outgrown moves over the cuts
+    _, capacity = capacity_until([1] * 5, [900, 1024, 1300, 40, 1700], 6, 8192, 0, 2040)
+    assert capacity.merge == 0 and capacity.work == 5
+    _, capacity = capacity_until([1] * 5, [900, 1024, 1300, 40, 1700], 6, 1000, 0, 2040)
+    assert capacity.merge_mid == 5 and capacity.work == 10
     _, capacity = capacity_until([1] * 5, [900, 1024, 1300, 40, 1700], 6, None, 0, 2300)
     assert capacity.merge_mid == 5 and capacity.work == 5 * 5  # 2,300 keys are five chunks of 512
     _, capacity = capacity_until([1] * 2, [8000, 100], 6, None, 0, 10000)
