@@ -51,10 +51,6 @@ class StepBatch:
     static: Any = None  # for a step that is captured and replayed: the fixed homes of such plans (`ops.StaticPlans`)
 
     @property
-    def max_q_len(self) -> int:
-        return max(self.q_lens) if self.q_lens else 0
-
-    @property
     def max_kv_len(self) -> int:
         return max(self.kv_lens) if self.kv_lens else 0
 

@@ -120,10 +120,6 @@ class Runtime:
     # about a tenth less time to stream them.  Whoever loads the model decides, from the memory there is.
     stream_copies: bool = False
 
-    @property
-    def is_float32(self) -> bool:
-        return self.act_dtype == torch.float32
-
 
 class Part:
     """Base of every part."""

@@ -42,16 +42,10 @@ class Sampler:
     def __init__(self, device: torch.device) -> None:
         self.device = device
 
-    def sample_on_device(
-        self, logits: torch.Tensor, temperatures: torch.Tensor, top_ps: torch.Tensor, uniforms: torch.Tensor
-    ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-        """The same with parameters and results on the device (float32 [R] each in; int32 tokens and
-        two float32 log-probabilities out): nothing waits for the host, so that the tokens can feed
-        the next step as they are."""
-        return ops.sample(logits, temperatures, top_ps, uniforms)
-
     def sample_packed(self, logits: torch.Tensor, temperatures: torch.Tensor, top_ps: torch.Tensor, uniforms: torch.Tensor) -> torch.Tensor:
-        """The same as one int32 tensor [3, R] (tokens, then the bits of the two log-probabilities), which
+        """One token per row of float32 `logits` [R, V] with parameters and results on the device (float32 [R]
+        each in): nothing waits for the host, so that the tokens can feed the next step as they are.  The result is
+        one int32 tensor [3, R] (tokens, then the bits of the two log-probabilities that `sample` returns), which
         goes to the host in one copy; `unpack` reads it there."""
         return ops.sample_packed(logits, temperatures, top_ps, uniforms)
 
